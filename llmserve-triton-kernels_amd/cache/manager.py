@@ -37,13 +37,15 @@ class CacheGroup:
         return isinstance(self.spec, PagedCacheSpec)
 
 
-def group_layers(cache_specs: list[PagedCacheSpec | StateCacheSpec | None]) -> list[CacheGroup]:
+def group_layers(cache_specs: list) -> list[CacheGroup]:
     """Groups for a list of needs, one per entry of the model's schedule (None: the entry keeps
-    nothing of its own)."""
+    nothing of its own; a tuple: the entry keeps several things, pages and a state for instance, each in
+    the group of its kind)."""
     by_spec: dict = {}
     for layer, spec in enumerate(cache_specs):
-        if spec is not None:
-            by_spec.setdefault(spec, []).append(layer)
+        for one in (spec if isinstance(spec, (tuple, list)) else (spec,)):
+            if one is not None:
+                by_spec.setdefault(one, []).append(layer)
     return [CacheGroup(g, spec, tuple(layers)) for g, (spec, layers) in enumerate(by_spec.items())]
 
 
@@ -62,11 +64,17 @@ class StepLayout:
     table_updates: dict[int, list[tuple[int, int, int]]] = field(default_factory=dict)
 
 
-def window_pages(window: int, step_tokens: int, block_size: int) -> int:
+def window_pages(window: int, step_tokens: int, block_size: int, keep_first: int = 0) -> int:
     """Most pages a request holds in a group that keeps `window` keys, when a step brings up to `step_tokens` of
     its tokens: the keys the portion's first query still sees, the portion itself, and one page more because
-    neither starts at a page's edge.  (Pages out of reach come back after the step that passed them.)"""
-    return -(-(window - 1 + step_tokens) // block_size) + 1
+    neither starts at a page's edge; beside them the pages of the first `keep_first` keys, which are never
+    given back.  (Pages out of reach come back after the step that passed them.)"""
+    return -(-(window - 1 + step_tokens) // block_size) + 1 + -(-keep_first // block_size)
+
+
+def bounded_pages(spec: PagedCacheSpec, step_tokens: int, block_size: int) -> int:
+    """`window_pages` for a group whose reach is bounded by a window, by chunks, or by both."""
+    return window_pages(spec.live_tokens(), step_tokens, block_size, spec.keep_first)
 
 
 class CacheManager:
@@ -86,7 +94,7 @@ class CacheManager:
         self.tables: dict[int, dict] = {g.group_id: {} for g in self.paged_groups}
         self.lengths: dict = {}
         self.slot_of: dict = {}
-        self._windowed = [g for g in self.paged_groups if g.spec.window is not None]
+        self._bounded = [g for g in self.paged_groups if g.spec.bounded]
         self._slot_alloc = BlockAllocator(max_seqs)
         self._fresh: set[int] = set()
 
@@ -109,10 +117,10 @@ class CacheManager:
         full = self.blocks_for(n_tokens)
         need = {}
         for g in self.paged_groups:
-            if g.spec.window is None or step_tokens is None:
+            if not g.spec.bounded or step_tokens is None:
                 need[g.group_id] = full
             else:
-                need[g.group_id] = min(full, window_pages(g.spec.window, step_tokens, self.block_size))
+                need[g.group_id] = min(full, bounded_pages(g.spec, step_tokens, self.block_size))
         return need
 
     def pages_owed(self, seq_id, new_tokens: int, step_tokens: int | None = None) -> dict[int, int]:
@@ -125,9 +133,9 @@ class CacheManager:
         for g in self.paged_groups:
             table = self.tables[g.group_id][seq_id]
             owed[g.group_id] = max(0, want - len(table))
-            if g.spec.window is not None and step_tokens is not None:
+            if g.spec.bounded and step_tokens is not None:
                 held = sum(1 for page in table if page >= 0)
-                most = window_pages(g.spec.window, min(step_tokens, max(new_tokens, 1)), self.block_size)
+                most = bounded_pages(g.spec, min(step_tokens, max(new_tokens, 1)), self.block_size)
                 owed[g.group_id] = min(owed[g.group_id], max(0, most - held))
         return owed
 
@@ -260,24 +268,26 @@ class CacheManager:
         return self.tables[group_id][seq_id]
 
     def release_passed(self, seq_ids) -> int:
-        """After a step: return the pages of windowed groups that no later query can reach.
+        """After a step: return the pages of windowed or chunked groups that no later query can reach.
 
-        The next query of a request of length `len` sits at position >= len and sees the keys
-        j > position - window, so a page is dead when its last key is <= len - window.
+        The next query of a request of length `len` sits at position >= len.  With a window it sees the keys
+        j > position - window, so a page is dead when its last key is <= len - window; with chunks it sees
+        keys of its own chunk only, so a page is dead when its last key lies before the chunk of position
+        `len`.  Pages that hold one of the first `keep_first` keys are never dead.
         Returns the number of pages given back.
         """
         bs, freed = self.block_size, 0
-        if not self._windowed:
+        if not self._bounded:
             return 0
-        for g in self._windowed:
-            window = g.spec.window
+        for g in self._bounded:
+            kept = -(-g.spec.keep_first // bs)  # pages [0, kept) hold keys every query sees
             for s in seq_ids:
                 if s not in self.lengths:
                     continue
                 table = self.tables[g.group_id][s]
-                dead_upto = (self.lengths[s] - window + 1) // bs  # pages [0, dead_upto) are out of reach
+                dead_upto = g.spec.dead_before(self.lengths[s]) // bs  # pages [kept, dead_upto) are out of reach
                 back = []
-                for i in range(min(max(dead_upto, 0), len(table))):
+                for i in range(kept, min(max(dead_upto, 0), len(table))):
                     if table[i] >= 0:
                         back.append(table[i])
                         table[i] = -1

@@ -14,7 +14,7 @@ from dataclasses import dataclass
 
 import torch
 
-from .manager import CacheGroup, window_pages
+from .manager import CacheGroup, bounded_pages
 
 
 @dataclass
@@ -37,7 +37,8 @@ class StateLayerCache:
 def page_bytes_of(group: CacheGroup, block_size: int, elem_size: int) -> int:
     """Bytes one page of a paged group costs over the group's layers (keys and values); L layers give the
     reference's 2*L*kv_heads*block_size*head_dim*elem (src/llmserve/kvcache/paged.py:221-227)."""
-    return 2 * len(group.layers) * group.spec.num_kv_heads * block_size * group.spec.head_dim * elem_size
+    s = group.spec
+    return len(group.layers) * block_size * elem_size * (s.num_kv_heads * s.head_dim + s.v_heads * s.v_dim)
 
 
 def page_bytes(groups: list[CacheGroup], block_size: int, elem_size: int) -> int:
@@ -70,7 +71,7 @@ def pool_sizes_for_budget(groups: list[CacheGroup], block_size: int, elem_size: 
     if not paged:
         return {}
     full = -(-longest // block_size)
-    need = {g.group_id: full if g.spec.window is None else min(full, window_pages(g.spec.window, step_tokens, block_size))
+    need = {g.group_id: min(full, bounded_pages(g.spec, step_tokens, block_size)) if g.spec.bounded else full
             for g in paged}
     per_request = sum(need[g.group_id] * page_bytes_of(g, block_size, elem_size) for g in paged)
     requests = min(float(max_seqs), (budget_bytes - fixed) / per_request)
@@ -95,20 +96,20 @@ class CacheStorage:
         self.tables: dict[int, torch.Tensor] = {}
         self.block_size = block_size
         self.num_blocks = num_blocks
-        self._owner: dict[int, tuple[int, int]] = {}  # layer -> (group, index in group)
+        self._owner: dict[int, list[tuple[int, int]]] = {}  # layer -> (group, index in group) of everything it keeps
         self.k: dict[int, torch.Tensor] = {}
         self.v: dict[int, torch.Tensor] = {}
         self.state: dict[int, torch.Tensor] = {}
         for g in groups:
             for i, layer in enumerate(g.layers):
-                self._owner[layer] = (g.group_id, i)
+                self._owner.setdefault(layer, []).append((g.group_id, i))
             n = len(g.layers)
             if g.paged:
                 s = g.spec
                 pages = num_blocks[g.group_id] if isinstance(num_blocks, dict) else num_blocks
                 self.k[g.group_id] = torch.zeros((n, pages, s.num_kv_heads, block_size, s.head_dim),
                                                  dtype=dtype, device=device)
-                self.v[g.group_id] = torch.zeros((n, pages, s.num_kv_heads, s.head_dim, block_size),
+                self.v[g.group_id] = torch.zeros((n, pages, s.v_heads, s.v_dim, block_size),
                                                  dtype=dtype, device=device)
                 self.tables[g.group_id] = torch.zeros((max_seqs, table_width), dtype=torch.int32, device=device)
             else:
@@ -121,14 +122,20 @@ class CacheStorage:
 
     def layer_cache(self, layer: int, source: int | None = None):
         """Cache view for entry `layer` of the model's schedule; with `source`, the storage of
-        that other entry, read-only."""
+        that other entry, read-only.  An entry that keeps several things (pages and a state) gets a tuple
+        of views, pages first."""
         owner = layer if source is None else source
         if owner not in self._owner:
             return None
-        gid, i = self._owner[owner]
-        if gid in self.k:
-            return PagedLayerCache(self.k[gid][i], self.v[gid][i], self.block_size, gid, store=source is None)
-        return StateLayerCache(self.state[gid][i], gid)
+        views = []
+        for gid, i in self._owner[owner]:
+            if gid in self.k:
+                views.append(PagedLayerCache(self.k[gid][i], self.v[gid][i], self.block_size, gid, store=source is None))
+            else:
+                views.append(StateLayerCache(self.state[gid][i], gid))
+        if len(views) == 1:
+            return views[0]
+        return tuple(sorted(views, key=lambda v: not isinstance(v, PagedLayerCache)))
 
     def clear_state(self, slots: list[int]) -> None:
         """Zero the state of freshly taken slots in every state group."""

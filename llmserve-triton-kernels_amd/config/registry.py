@@ -74,6 +74,8 @@ def architecture_of(config_dict: dict) -> Architecture:
     names = config_dict.get("architectures")
     if names:
         name = names[0]
+    elif isinstance(config_dict.get("architecture"), str):  # (some configurations name their one architecture so)
+        name = config_dict["architecture"]
     elif config_dict.get("model_type") in _MODEL_TYPES:
         name = _MODEL_TYPES[config_dict["model_type"]]
     else:

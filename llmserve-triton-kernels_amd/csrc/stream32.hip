@@ -1,0 +1,102 @@
+// Kernels of a layer whose residual stream is kept in 32-bit whatever the model's dtype:
+//   embed_scale      x[n] = table[ids[n]] * scale                                   (table T, x float)
+//   rmsnorm32        y[r] = x[s] * rsqrt(mean(x[s]^2) + eps) * (offset + w), s = rows[r] or r   (x float, y T)
+//   gated_add        x[n] += sum over branches b of g_b * y_b[n]                    (all float)
+//                    g_b = sigmoid(z_b[n] + bias_b) where the branch has a gate, else 1
+// T is float or bfloat16.  One workgroup per row; every reduction has an order fixed by the sizes alone.
+#include "common.h"
+
+#define S32_THREADS 256
+
+template <typename T>
+__global__ __launch_bounds__(S32_THREADS) void embed_scale_kernel(float* __restrict__ out, const T* __restrict__ table,
+                                                                  const int* __restrict__ ids, int hidden, int vocab,
+                                                                  float scale) {
+    const int n = blockIdx.x;
+    int id = ids[n];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+    const T* row = table + (size_t)id * hidden;
+    for (int c = threadIdx.x; c < hidden; c += S32_THREADS) out[(size_t)n * hidden + c] = to_f32(row[c]) * scale;
+}
+
+template <typename T>
+__global__ __launch_bounds__(S32_THREADS) void rmsnorm32_kernel(T* __restrict__ out, const float* __restrict__ x,
+                                                                const float* __restrict__ weight,
+                                                                const int* __restrict__ rows, int hidden, float eps,
+                                                                float offset) {
+    __shared__ float lds[16];
+    const int r = blockIdx.x;
+    const float* xr = x + (size_t)(rows ? rows[r] : r) * hidden;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < hidden; c += S32_THREADS) {
+        const float v = xr[c];
+        ss = fmaf(v, v, ss);
+    }
+    const float inv = 1.0f / sqrtf(block_sum(ss, lds) / (float)hidden + eps);
+    for (int c = threadIdx.x; c < hidden; c += S32_THREADS)
+        out[(size_t)r * hidden + c] = from_f32<T>(xr[c] * inv * (offset + weight[c]));
+}
+
+// z: [N, z_stride] raw gate products, branch b's at columns z_col[b] .. z_col[b] + hidden (z_col[b] < 0: no gate).
+__global__ __launch_bounds__(S32_THREADS) void gated_add_kernel(float* __restrict__ x, const float* __restrict__ z,
+                                                                int z_stride, int z_col0, int z_col1,
+                                                                const float* __restrict__ bias0,
+                                                                const float* __restrict__ bias1,
+                                                                const float* __restrict__ y0, int y0_stride,
+                                                                const float* __restrict__ y1, int y1_stride,
+                                                                int hidden) {
+    const int n = blockIdx.x;
+    for (int c = threadIdx.x; c < hidden; c += S32_THREADS) {
+        float sum = 0.f;
+        if (y0) {
+            float g = 1.f;
+            if (z_col0 >= 0) g = 1.f / (1.f + expf(-(z[(size_t)n * z_stride + z_col0 + c] + (bias0 ? bias0[c] : 0.f))));
+            sum = g * y0[(size_t)n * y0_stride + c];
+        }
+        if (y1) {
+            float g = 1.f;
+            if (z_col1 >= 0) g = 1.f / (1.f + expf(-(z[(size_t)n * z_stride + z_col1 + c] + (bias1 ? bias1[c] : 0.f))));
+            sum += g * y1[(size_t)n * y1_stride + c];
+        }
+        x[(size_t)n * hidden + c] += sum;
+    }
+}
+
+extern "C" {
+
+int llms_embed_scale(int dtype, float* out, const void* table, const int* ids, int n, int hidden, int vocab, float scale,
+                     hipStream_t stream) {
+    LLMS_REQUIRE(n > 0 && hidden > 0 && vocab > 0, "embed_scale: sizes must be positive");
+    if (dtype == 0)
+        embed_scale_kernel<float><<<n, S32_THREADS, 0, stream>>>(out, (const float*)table, ids, hidden, vocab, scale);
+    else if (dtype == 1)
+        embed_scale_kernel<bf16><<<n, S32_THREADS, 0, stream>>>(out, (const bf16*)table, ids, hidden, vocab, scale);
+    else
+        LLMS_REQUIRE(false, "embed_scale: dtype must be 0 (float32) or 1 (bfloat16)");
+    LLMS_LAUNCH_CHECK();
+}
+
+int llms_rmsnorm32(int dtype, void* out, const float* x, const float* weight, const int* rows, float eps, float offset,
+                   int n_out, int hidden, hipStream_t stream) {
+    LLMS_REQUIRE(n_out > 0 && hidden > 0, "rmsnorm32: sizes must be positive");
+    if (dtype == 0)
+        rmsnorm32_kernel<float><<<n_out, S32_THREADS, 0, stream>>>((float*)out, x, weight, rows, hidden, eps, offset);
+    else if (dtype == 1)
+        rmsnorm32_kernel<bf16><<<n_out, S32_THREADS, 0, stream>>>((bf16*)out, x, weight, rows, hidden, eps, offset);
+    else
+        LLMS_REQUIRE(false, "rmsnorm32: dtype must be 0 (float32) or 1 (bfloat16)");
+    LLMS_LAUNCH_CHECK();
+}
+
+int llms_gated_add(float* x, const float* z, int z_stride, int z_col0, int z_col1, const float* bias0,
+                   const float* bias1, const float* y0, int y0_stride, const float* y1, int y1_stride, int n,
+                   int hidden, hipStream_t stream) {
+    LLMS_REQUIRE(n > 0 && hidden > 0, "gated_add: sizes must be positive");
+    LLMS_REQUIRE(y0 || y1, "gated_add: no branch to add");
+    LLMS_REQUIRE(z || (z_col0 < 0 && z_col1 < 0), "gated_add: gate columns named without gate products");
+    gated_add_kernel<<<n, S32_THREADS, 0, stream>>>(x, z, z_stride, z_col0, z_col1, bias0, bias1, y0, y0_stride, y1,
+                                                    y1_stride, hidden);
+    LLMS_LAUNCH_CHECK();
+}
+
+}  // extern "C"

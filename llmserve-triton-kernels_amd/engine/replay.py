@@ -47,7 +47,7 @@ def main(argv=None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time (each rounded up to a multiple of 64)")
     ap.add_argument("--block-size", type=int, default=16, help="tokens in a cache page")
-    ap.add_argument("--max-seqs", type=int, default=8, help="most requests alive at once")
+    ap.add_argument("--max-seqs", type=int, default=4, help="most requests alive at once (state slots)")
     args = ap.parse_args(argv)
 
     import numpy as np

@@ -107,6 +107,7 @@ class ModelRunner:
         model = Model(arch.build_spec(config), BuildContext(dtype, device))
         infos = model.param_infos()
         ignore = {model.spec.weights["head"] + "weight"} if getattr(model.head, "tied", False) else set()
+        ignore |= set(model.spec.unused_tensors)
         model.load(load_tensors(model_dir, infos, dtype, device, ignore))
         return cls(model, config, engine_config, device)
 

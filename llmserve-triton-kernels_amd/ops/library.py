@@ -732,6 +732,232 @@ def attention_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_p
     return out
 
 
+# ------------------------------------------------------------------------------ a residual stream in 32-bit
+
+
+def embed_scale(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, scale: float) -> torch.Tensor:
+    """out[n] = table[ids[n]] * scale in 32-bit; out float32 [N, H], table [V, H] float32 or bfloat16."""
+    dev = _dev(out, table, ids)
+    _rows(out, "out")
+    _rows(table, "table", out.shape[1])
+    _i32(ids, "ids", out.shape[0])
+    if out.dtype != torch.float32:
+        raise ValueError("out must be float32")
+    if out.shape[0] == 0:
+        return out
+    _check(load("stream32").llms_embed_scale(
+        c_int(_code(table)), _ptr(out), _ptr(table), _ptr(ids), c_int(out.shape[0]), c_int(out.shape[1]),
+        c_int(table.shape[0]), c_float(scale), _stream(dev)), "embed_scale")
+    return out
+
+
+def rmsnorm32(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float, offset: float = 0.0,
+              rows: torch.Tensor | None = None) -> torch.Tensor:
+    """out[r] = x[s] / sqrt(mean(x[s]^2) + eps) * (offset + weight), s = rows[r] or r, all in 32-bit and rounded
+    once; x and weight float32, out float32 or bfloat16."""
+    dev = _dev(out, x, weight, rows)
+    _rows(x, "x")
+    hidden = x.shape[1]
+    _rows(out, "out", hidden)
+    _f32(weight, "weight", hidden)
+    if x.dtype != torch.float32:
+        raise ValueError("x must be float32")
+    if rows is not None:
+        _i32(rows, "rows", out.shape[0])
+    elif out.shape[0] != x.shape[0]:
+        raise ValueError("out and x differ in rows")
+    if out.shape[0] == 0:
+        return out
+    _check(load("stream32").llms_rmsnorm32(
+        c_int(_code(out)), _ptr(out), _ptr(x), _ptr(weight), _ptr(rows), c_float(eps), c_float(offset),
+        c_int(out.shape[0]), c_int(hidden), _stream(dev)), "rmsnorm32")
+    return out
+
+
+def gated_add(x: torch.Tensor, branches: list, gate_products: torch.Tensor | None = None) -> torch.Tensor:
+    """x += sum over up to two branches of g * y, in place, all float32.  A branch is (y [N, hidden], column, bias):
+    g = sigmoid(gate_products[:, column : column + hidden] + bias) where `column` is not None, else 1."""
+    ys = [b for b in branches if b is not None]
+    if not 1 <= len(ys) <= 2:
+        raise ValueError("one or two branches")
+    dev = _dev(x, gate_products, *[t for y, _c, bias in ys for t in (y, bias)])
+    _rows(x, "x")
+    n, hidden = x.shape
+    if x.dtype != torch.float32:
+        raise ValueError("x must be float32")
+    z_stride = 0
+    if gate_products is not None:
+        if gate_products.dim() != 2 or gate_products.stride(1) != 1 or gate_products.dtype != torch.float32 \
+                or gate_products.shape[0] != n:
+            raise ValueError("gate_products must be float32 [N, columns] with unit inner stride")
+        z_stride = gate_products.stride(0)
+    args = []
+    for y, column, bias in ys + [(None, None, None)] * (2 - len(ys)):
+        if y is not None:
+            if y.dim() != 2 or y.stride(1) != 1 or y.dtype != torch.float32 or tuple(y.shape) != (n, hidden):
+                raise ValueError("a branch must be float32 [N, hidden] with unit inner stride")
+            if column is not None:
+                if gate_products is None or not 0 <= column <= gate_products.shape[1] - hidden:
+                    raise ValueError("a gate's columns lie outside gate_products")
+                if bias is not None:
+                    _f32(bias, "bias", hidden)
+        args.append((y, -1 if column is None else column, bias if column is not None else None))
+    if n == 0:
+        return x
+    (y0, c0, b0), (y1, c1, b1) = args
+    _check(load("stream32").llms_gated_add(
+        _ptr(x), _ptr(gate_products), c_int(z_stride), c_int(c0), c_int(c1), _ptr(b0), _ptr(b1), _ptr(y0),
+        c_int(y0.stride(0) if y0 is not None else 0), _ptr(y1), c_int(y1.stride(0) if y1 is not None else 0),
+        c_int(n), c_int(hidden), _stream(dev)), "gated_add")
+    return x
+
+
+# ------------------------------------------------------------------------------ attention from chosen ingredients
+
+
+def conv_store(q_out: torch.Tensor, proj: torch.Tensor, *, cq: int, k_heads: int, dk: int, v_heads: int, dv: int,
+               taps_w: torch.Tensor | None = None, state: torch.Tensor | None = None,
+               state_slots: torch.Tensor | None = None, token_seq: torch.Tensor | None = None,
+               positions: torch.Tensor | None = None, cu_seqlens: torch.Tensor | None = None,
+               slots: torch.Tensor | None = None, k_pool: torch.Tensor | None = None,
+               v_pool: torch.Tensor | None = None, block_size: int = 0) -> torch.Tensor:
+    """proj float32 [N, cq + k_heads*dk + v_heads*dv] (what the stacked q, k, v projection gave), optionally through a
+    causal convolution per channel (`taps_w` float32 [channels, taps], `state` float32 [slots, taps-1, channels]: a
+    ring of each request's last projected rows, indexed by position), rounded once: queries to q_out [N, cq], keys
+    and values to the tokens' cache slots (`slots`; None: nothing is stored)."""
+    dev = _dev(q_out, proj, taps_w, state, state_slots, token_seq, positions, cu_seqlens, slots, k_pool, v_pool)
+    n = proj.shape[0]
+    channels = cq + k_heads * dk + v_heads * dv
+    if proj.dim() != 2 or proj.dtype != torch.float32 or proj.stride(1) != 1 or proj.shape[1] != channels:
+        raise ValueError(f"proj must be float32 [N, {channels}] with unit inner stride")
+    _rows(q_out, "q_out", cq)
+    if q_out.shape[0] != n:
+        raise ValueError("q_out and proj differ in rows")
+    taps = 0
+    if taps_w is not None:
+        _f32(taps_w, "taps_w")
+        if taps_w.dim() != 2 or taps_w.shape[0] != channels:
+            raise ValueError(f"taps_w must be [{channels}, taps]")
+        taps = taps_w.shape[1]
+    if taps > 0:
+        _i32(token_seq, "token_seq", n)
+        _i32(positions, "positions", n)
+        _i32(cu_seqlens, "cu_seqlens")
+    if taps > 1:
+        if state is None or state.dtype != torch.float32 or not state.is_contiguous() or \
+                tuple(state.shape[1:]) != (taps - 1, channels):
+            raise ValueError(f"state must be a contiguous float32 [slots, {taps - 1}, {channels}] tensor")
+        _i32(state_slots, "state_slots", cu_seqlens.numel() - 1)
+    if slots is not None:
+        _i32(slots, "slots", n)
+        pages = k_pool.shape[0]
+        if tuple(k_pool.shape) != (pages, k_heads, block_size, dk) or not k_pool.is_contiguous():
+            raise ValueError(f"k_pool shape {tuple(k_pool.shape)} is not [pages,{k_heads},{block_size},{dk}]")
+        if tuple(v_pool.shape) != (pages, v_heads, dv, block_size) or not v_pool.is_contiguous():
+            raise ValueError(f"v_pool shape {tuple(v_pool.shape)} is not [pages,{v_heads},{dv},{block_size}]")
+        if k_pool.dtype != q_out.dtype or v_pool.dtype != q_out.dtype:
+            raise ValueError("pools and q_out differ in dtype")
+    if n == 0:
+        return q_out
+    _check(load("attention_composed").llms_conv_store(
+        c_int(_code(q_out)), _ptr(q_out), c_int(q_out.stride(0)), _ptr(proj), c_int(proj.stride(0)), _ptr(taps_w),
+        c_int(taps), _ptr(state), ctypes.c_size_t(state.stride(0) if state is not None else 0), _ptr(state_slots),
+        _ptr(token_seq), _ptr(positions), _ptr(cu_seqlens), _ptr(slots), _ptr(k_pool), _ptr(v_pool), c_int(n), c_int(cq),
+        c_int(k_heads * dk), c_int(v_heads * dv), c_int(k_heads), c_int(dk), c_int(v_heads), c_int(dv),
+        c_int(block_size), _stream(dev)), "conv_store")
+    return q_out
+
+
+def conv_state(state: torch.Tensor, proj: torch.Tensor, state_slots: torch.Tensor, cu_seqlens: torch.Tensor,
+               context_lens: torch.Tensor) -> None:
+    """The ring `state` [slots, taps-1, channels] takes the last taps-1 rows of `proj` of every request of the step
+    (request b owns rows cu_seqlens[b] .. cu_seqlens[b+1] and is context_lens[b] long after the step; a request
+    of length 0 is padding and left alone)."""
+    dev = _dev(state, proj, state_slots, cu_seqlens, context_lens)
+    if state.dtype != torch.float32 or state.dim() != 3 or not state.is_contiguous():
+        raise ValueError("state must be a contiguous float32 [slots, taps-1, channels] tensor")
+    channels = state.shape[2]
+    if proj.dim() != 2 or proj.dtype != torch.float32 or proj.stride(1) != 1 or proj.shape[1] != channels:
+        raise ValueError(f"proj must be float32 [N, {channels}] with unit inner stride")
+    _i32(cu_seqlens, "cu_seqlens")
+    b = cu_seqlens.numel() - 1
+    _i32(context_lens, "context_lens", b)
+    _i32(state_slots, "state_slots", b)
+    if b <= 0 or proj.shape[0] == 0:
+        return
+    _check(load("attention_composed").llms_conv_state(
+        _ptr(state), ctypes.c_size_t(state.stride(0)), _ptr(state_slots), _ptr(proj), c_int(proj.stride(0)),
+        _ptr(cu_seqlens), _ptr(context_lens), c_int(b), c_int(state.shape[1] + 1), c_int(channels), _stream(dev)),
+        "conv_state")
+
+
+ATTEND_COMPOSED_LDS = 160 * 1024
+
+
+def attend_composed_lds_bytes(heads: int, maps: int, dk: int, dv: int, talk: bool) -> int:
+    """LDS one workgroup of `attend_composed` takes."""
+    s = heads * maps
+    floats = s * dk + 2 * s + s * 64 + s * dv + ((heads * 64 + heads * heads) if talk else 0)
+    return floats * 4 + 2 * 64 * 4
+
+
+def attend_composed(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                    block_tables: torch.Tensor, token_seq: torch.Tensor, positions: torch.Tensor, *, heads: int,
+                    kv_heads: int, dk: int, dv: int, block_size: int, scale: float, maps: int = 1, window: int = 0,
+                    keep_first: int = 0, chunk: int = 0, slopes: torch.Tensor | None = None,
+                    talk: torch.Tensor | None = None, lam: float = 0.0, head_norm: bool = False, eps: float = 0.0,
+                    out_scale: float = 1.0, table_rows: torch.Tensor | None = None,
+                    context_lens: torch.Tensor | None = None) -> torch.Tensor:
+    """Attention of N new tokens over the paged cache, one workgroup per token (all its heads), float32 or bfloat16
+    storage, 32-bit arithmetic.  q [N, heads*maps*dk] (head by head, a head's maps side by side); k_pool
+    [pages, kv_heads*maps, block, dk]; v_pool [pages, kv_heads, dv, block]; out [N, heads*dv].  A query at
+    position i sees j <= i with j >= its chunk's start (chunk > 0) and (i - j < window or j < keep_first) (window >
+    0).  `slopes` float32 [heads]: slope_h * (i - j) is taken off the scores.  `talk` float32 [heads, heads]: the
+    heads' normalised weights are mixed, w_h = sum_g talk[h, g] w_g (maps = 1).  maps = 2: a_1 - lam * a_2.
+    `head_norm`: each head's result is divided by its root mean square (eps inside the root) and multiplied by
+    out_scale.  `context_lens` [B]: rows of a request of length 0 are padding and give zeros."""
+    dev = _dev(out, q, k_pool, v_pool, block_tables, token_seq, positions, slopes, talk, table_rows, context_lens)
+    n = q.shape[0]
+    if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < heads * maps * dk:
+        raise ValueError("q must be [N, >= heads*maps*dk] with unit inner stride")
+    _rows(out, "out", heads * dv)
+    if out.shape[0] != n or out.dtype != q.dtype:
+        raise ValueError("out and q disagree")
+    pages = k_pool.shape[0]
+    if tuple(k_pool.shape) != (pages, kv_heads * maps, block_size, dk) or not k_pool.is_contiguous():
+        raise ValueError(f"k_pool shape {tuple(k_pool.shape)} is not [pages,{kv_heads * maps},{block_size},{dk}]")
+    if tuple(v_pool.shape) != (pages, kv_heads, dv, block_size) or not v_pool.is_contiguous():
+        raise ValueError(f"v_pool shape {tuple(v_pool.shape)} is not [pages,{kv_heads},{dv},{block_size}]")
+    if k_pool.dtype != q.dtype or v_pool.dtype != q.dtype:
+        raise ValueError("pools and q differ in dtype")
+    if block_tables.dim() != 2 or block_tables.dtype != torch.int32 or not block_tables.is_contiguous():
+        raise ValueError("block_tables must be a contiguous int32 [B, M] tensor")
+    if heads % kv_heads or maps not in (1, 2) or (talk is not None and maps != 1):
+        raise ValueError("heads must be a multiple of kv_heads, maps 1 or 2, and talk goes with maps = 1")
+    _i32(token_seq, "token_seq", n)
+    _i32(positions, "positions", n)
+    if table_rows is not None:
+        _i32(table_rows, "table_rows")
+    if context_lens is not None:
+        _i32(context_lens, "context_lens")
+    if slopes is not None:
+        _f32(slopes, "slopes", heads)
+    if talk is not None:
+        _f32(talk, "talk", heads * heads)
+    if attend_composed_lds_bytes(heads, maps, dk, dv, talk is not None) > ATTEND_COMPOSED_LDS:
+        raise ValueError("heads times sizes do not fit the 160 KB of LDS a workgroup has")
+    if n == 0:
+        return out
+    _check(load("attention_composed").llms_attend_composed(
+        c_int(_code(q)), _ptr(out), c_int(out.stride(0)), _ptr(q), c_int(q.stride(0)), _ptr(k_pool), _ptr(v_pool),
+        _ptr(block_tables), _ptr(table_rows), c_int(block_tables.shape[1]), _ptr(token_seq), _ptr(positions),
+        _ptr(context_lens), c_int(n), c_int(heads), c_int(kv_heads), c_int(maps), c_int(dk), c_int(dv),
+        c_int(block_size), c_int(window), c_int(keep_first), c_int(chunk), c_float(scale), _ptr(slopes), _ptr(talk),
+        c_float(lam), c_int(1 if head_norm else 0), c_float(eps), c_float(out_scale), _stream(dev)),
+        "attend_composed")
+    return out
+
+
 # ------------------------------------------------------------------------------ sampling
 
 

@@ -1,0 +1,165 @@
+"""Attention put together from ingredients that its parameters choose, over the paged cache.
+
+Parameters (a `PartSpec` of kind "composed_attention"):
+  hidden, num_heads (H), num_kv_heads (G), head_dim (dk, of queries and keys), value_dim (dv; default dk),
+  scale                 the scores' factor (default 1 / sqrt(dk))
+  window, keep_first    a query at i sees j <= i with i - j < window, and beside them the keys j < keep_first
+                        (window None: every earlier key)
+  chunk                 a query sees only keys of its own run of `chunk` positions, counted from position 0
+  conv_taps             a causal convolution over time on every channel of q, k and v, directly behind the
+                        projection: y_t = sum_j w[:, j] u_(t - taps + 1 + j), zeros before the sequence (0: none).
+                        The last taps - 1 projected rows of a request are its state.
+  distance_slope_base   b: slope_h * (i - j) is taken off the scores, slope_h = 2^(-b (h + 1) / H)  (None: no bias)
+  talking_heads         the heads' softmax weights are mixed before they meet the values: w_h = sum_g T[h, g] w_g,
+                        head h applying its mixed weights to the values of its own key/value head
+  differential          two score maps per head over the same values (q and k hold [map 1, map 2] head by head),
+                        o = a_1 - lambda a_2 with lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + `diff`
+  head_norm_eps         each head's result is divided by its root mean square (eps inside the root), no weight,
+                        and multiplied by `head_norm_scale` (None: no such norm)
+  result                "float32": the output projection's result stays unrounded (for a 32-bit residual stream)
+  names                 local tensor names (defaults: q, k, v, o, q.conv, k.conv, v.conv, talk, lq1, lk1, lq2, lk2)
+
+Scores, softmax, the mixing of heads, the difference of the maps and the head norm are computed in 32-bit; the
+convolution is computed in 32-bit from the unrounded projection and rounded once.  Keys are cached as [pages,
+G * maps, block, dk] and values as [pages, G, dv, block]; a windowed or chunked layer gives the pages that no
+later query can reach back while the request runs.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from ..ops import library as ops
+from .linear import linear
+from .registry import Mixer, register_mixer
+from .spec import PagedCacheSpec, ParamInfo, StateCacheSpec
+
+_DEFAULT_NAMES = {"q": "q", "k": "k", "v": "v", "o": "o", "q_conv": "q.conv", "k_conv": "k.conv", "v_conv": "v.conv",
+                  "talk": "talk", "lq1": "lq1", "lk1": "lk1", "lq2": "lq2", "lk2": "lk2"}
+
+
+def _fill_taps(shape, generator, device, options):
+    """Taps of a short convolution: the newest tap near one, the older ones smaller."""
+    w = 0.3 * torch.randn(shape, generator=generator, dtype=torch.float32, device=device)
+    w[:, -1] += 1.0
+    return w
+
+
+def _fill_talk(shape, generator, device, options):
+    """A mixing matrix of heads: near the identity."""
+    w = 0.2 * torch.randn(shape, generator=generator, dtype=torch.float32, device=device)
+    return w + torch.eye(shape[0], dtype=torch.float32, device=device)
+
+
+@register_mixer("composed_attention")
+class ComposedAttention(Mixer):
+    graph_safe = True
+
+    def __init__(self, spec, ctx):
+        super().__init__(spec, ctx)
+        self.hidden = int(spec["hidden"])
+        self.num_heads = int(spec["num_heads"])
+        self.num_kv_heads = int(spec["num_kv_heads"])
+        self.head_dim = int(spec["head_dim"])
+        self.value_dim = int(spec.get("value_dim") or self.head_dim)
+        self.scale = float(spec["scale"]) if spec.get("scale") is not None else 1.0 / math.sqrt(self.head_dim)
+        self.window = spec.get("window")
+        self.keep_first = int(spec.get("keep_first") or 0) if self.window is not None else 0
+        self.chunk = spec.get("chunk")
+        self.taps = int(spec.get("conv_taps") or 0)
+        self.slope_base = spec.get("distance_slope_base")
+        self.talking = bool(spec.get("talking_heads", False))
+        self.differential = bool(spec.get("differential", False))
+        self.diff = float(spec.get("diff", 0.0))
+        self.head_norm_eps = spec.get("head_norm_eps")
+        self.head_norm_scale = float(spec.get("head_norm_scale", 1.0))
+        self.result_dtype = torch.float32 if spec.get("result", "model") == "float32" else None
+        self.names = dict(_DEFAULT_NAMES, **(spec.get("names") or {}))
+        self.maps = 2 if self.differential else 1
+        if self.num_heads % self.num_kv_heads:
+            raise ValueError("num_heads must be a multiple of num_kv_heads")
+        for name in ("window", "chunk"):
+            value = getattr(self, name)
+            if value is not None and int(value) < 1:
+                raise ValueError(f"{name} must be >= 1")
+        if self.talking and self.differential:
+            raise ValueError("mixing the heads' weights and two score maps per head do not go together")
+        lds = ops.attend_composed_lds_bytes(self.num_heads, self.maps, self.head_dim, self.value_dim, self.talking)
+        if lds > ops.ATTEND_COMPOSED_LDS:
+            raise ValueError(f"{self.num_heads} heads of sizes {self.head_dim} and {self.value_dim} need {lds} bytes "
+                             f"of LDS per token; the kernel has {ops.ATTEND_COMPOSED_LDS}")
+        self.cq = self.num_heads * self.maps * self.head_dim
+        self.ck = self.num_kv_heads * self.maps * self.head_dim
+        self.cv = self.num_kv_heads * self.value_dim
+        self.qkv_weight = self.o_weight = self.taps_w = self.talk = self.slopes = None
+        self.lam = 0.0
+
+    # ---- what it keeps between steps -------------------------------------------------------------
+    def cache_spec(self):
+        paged = PagedCacheSpec(num_kv_heads=self.num_kv_heads * self.maps, head_dim=self.head_dim,
+                               window=None if self.window is None else int(self.window), keep_first=self.keep_first,
+                               chunk=None if self.chunk is None else int(self.chunk),
+                               value_heads=self.num_kv_heads, value_dim=self.value_dim)
+        if self.taps > 1:
+            return (paged, StateCacheSpec((self.taps - 1, self.cq + self.ck + self.cv), "float32"))
+        return paged
+
+    # ---- tensors -----------------------------------------------------------------------------------
+    def param_infos(self):
+        n, h = self.names, self.hidden
+        infos = {n["q"]: ParamInfo((self.cq, h)), n["k"]: ParamInfo((self.ck, h)), n["v"]: ParamInfo((self.cv, h)),
+                 n["o"]: ParamInfo((h, self.num_heads * self.value_dim))}
+        if self.taps > 0:
+            for key, channels in (("q_conv", self.cq), ("k_conv", self.ck), ("v_conv", self.cv)):
+                infos[n[key]] = ParamInfo((channels, self.taps), _fill_taps)
+        if self.talking:
+            infos[n["talk"]] = ParamInfo((self.num_heads, self.num_heads), _fill_talk)
+        if self.differential:
+            for key in ("lq1", "lk1", "lq2", "lk2"):
+                infos[n[key]] = ParamInfo((self.head_dim,), "around_zero")
+        return infos
+
+    def load(self, tensors):
+        n = self.names
+        dev = tensors[n["q"]].device
+        self.qkv_weight = torch.cat([tensors[n[x]] for x in "qkv"], dim=0).contiguous()
+        self.o_weight = tensors[n["o"]].contiguous()
+        if self.taps > 0:
+            self.taps_w = torch.cat([tensors[n[x + "_conv"]].float() for x in "qkv"], dim=0).contiguous()
+        if self.talking:
+            self.talk = tensors[n["talk"]].float().contiguous()
+        if self.slope_base is not None:
+            heads = self.num_heads
+            self.slopes = torch.tensor([2.0 ** (-float(self.slope_base) * (i + 1) / heads) for i in range(heads)],
+                                       dtype=torch.float32, device=dev)
+        if self.differential:  # one number for the layer, worked out once
+            dot = [float((tensors[n[a]].double() * tensors[n[b]].double()).sum()) for a, b in (("lq1", "lk1"), ("lq2", "lk2"))]
+            self.lam = math.exp(dot[0]) - math.exp(dot[1]) + self.diff
+
+    # ---- one step ------------------------------------------------------------------------------------
+    def forward(self, x, batch, cache):
+        paged, state = cache if isinstance(cache, tuple) else (cache, None)
+        view = batch.groups[paged.group_id]
+        heads, kv, dk, dv = self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim
+        proj = linear(x, self.qkv_weight, out_dtype=torch.float32)  # q, k and v side by side, unrounded
+        q = torch.empty((proj.shape[0], self.cq), dtype=x.dtype, device=x.device)
+        conv, taps = self.taps > 1, self.taps > 0  # (one tap is a factor per channel and needs no state)
+        ops.conv_store(q, proj, cq=self.cq, k_heads=kv * self.maps, dk=dk, v_heads=kv, dv=dv,
+                       taps_w=self.taps_w if taps else None,
+                       state=state.state if conv else None, state_slots=batch.state_slots if conv else None,
+                       token_seq=batch.token_seq if taps else None, positions=batch.positions if taps else None,
+                       cu_seqlens=batch.cu_seqlens if taps else None, slots=view.slots if paged.store else None,
+                       k_pool=paged.k_pool, v_pool=paged.v_pool, block_size=paged.block_size)
+        if conv:
+            ops.conv_state(state.state, proj, batch.state_slots, batch.cu_seqlens, batch.context_lens)
+        out = torch.empty((proj.shape[0], heads * dv), dtype=x.dtype, device=x.device)
+        ops.attend_composed(out, q, paged.k_pool, paged.v_pool, view.block_tables, batch.token_seq, batch.positions,
+                            heads=heads, kv_heads=kv, dk=dk, dv=dv, block_size=paged.block_size, scale=self.scale,
+                            maps=self.maps, window=int(self.window or 0), keep_first=self.keep_first,
+                            chunk=int(self.chunk or 0), slopes=self.slopes, talk=self.talk, lam=self.lam,
+                            head_norm=self.head_norm_eps is not None, eps=float(self.head_norm_eps or 0.0),
+                            out_scale=self.head_norm_scale, table_rows=batch.state_slots,
+                            context_lens=batch.context_lens)
+        return linear(out, self.o_weight, out_dtype=self.result_dtype)

@@ -1,5 +1,11 @@
 """Arrangements of a layer's parts.
 
+"parallel" has one norm that both branches read: with h = norm(x),
+    x = x + g_mixer * mixer(h) + g_feed_forward * feed_forward(h)
+where each g is the branch's gate (a part of the family "gate"; kind "none": no gate) and the residual
+stream x is 32-bit whatever the model's dtype: the branches' results arrive unrounded and one kernel
+applies the gates and sums.
+
 "prenorm" is the reference's decoder layer (src/llmserve/model/llama.py:131-135):
     x = x + mixer(norm1(x));  x = x + feed_forward(norm2(x))
 The hidden state travels as (x, delta) with the last sum still open, so each residual
@@ -8,6 +14,10 @@ sum is done, in 32-bit, by the norm kernel that needs its result.
 
 from __future__ import annotations
 
+import torch
+
+from ..ops import library as ops
+from .linear import linear
 from .registry import ADDED_IN_PLACE, Block, DeferredNorm, register_block
 
 
@@ -25,3 +35,45 @@ class PreNormBlock(Block):
         if not h2.resolved:
             raise RuntimeError(f"{type(self.feed_forward).__name__} took a deferred input and left it unresolved")
         return h2.residual, None if f is ADDED_IN_PLACE else f
+
+
+@register_block("parallel")
+class ParallelBlock(Block):
+    """One norm, two branches beside each other, each with a gate of its own; a 32-bit residual stream, summed in
+    place.  The feed-forward may be of kind "none" (the layer has a mixer only)."""
+
+    ROLES = {"mixer": "mixer", "feed_forward": "feed_forward", "norm": "norm", "mixer_gate": "gate",
+             "feed_forward_gate": "gate"}
+
+    def __init__(self, parts):
+        super().__init__(parts)
+        self._stacked = None  # the two gates' weights as one matrix, made at the first step
+
+    def _gate_products(self, h):
+        """(products [N, columns] or None, column of the mixer's gate or None, column of the feed-forward's)."""
+        gm, gf = self.mixer_gate, self.feed_forward_gate
+        wm, wf = gm.weight, gf.weight
+        if wm is not None and wf is not None:  # one product for both
+            if self._stacked is None:
+                self._stacked = torch.cat([wm, wf], dim=0).contiguous()
+            return linear(h, self._stacked, out_dtype=torch.float32), 0, wm.shape[0]
+        zm, zf = gm.products(h), gf.products(h)
+        if zm is not None and zf is not None:
+            return torch.cat([zm, zf], dim=1), 0, zm.shape[1]
+        one = zm if zm is not None else zf
+        return one, (0 if zm is not None else None), (0 if zf is not None else None)
+
+    def forward(self, x, delta, batch, cache):
+        if delta is not None or x.dtype != torch.float32:
+            raise ValueError("the parallel arrangement keeps a closed 32-bit residual stream")
+        h = self.norm.forward(x)
+        z, col_m, col_f = self._gate_products(h)
+        a = self.mixer.forward(h, batch, cache)
+        f = self.feed_forward.forward(h)
+        branches = []
+        for y, col, gate in ((a, col_m, self.mixer_gate), (f, col_f, self.feed_forward_gate)):
+            if y is not None:
+                branches.append((y if y.dtype == torch.float32 else y.float(), col, gate.bias))
+        if branches:
+            ops.gated_add(x, branches, z)
+        return x, None

@@ -20,15 +20,27 @@ class TokenEmbedding(Part):
         super().__init__(spec, ctx)
         self.vocab = int(spec["vocab"])
         self.hidden = int(spec["hidden"])
+        # `scale`: the row is multiplied by it; `stream`: "float32" starts a residual stream that is kept in 32-bit
+        # whatever the model's dtype (the product is then formed in 32-bit as well); `tensor`: the table's local name
+        self.scale = spec.get("scale")
+        self.stream = spec.get("stream", "model")
+        self.tensor = spec.get("tensor", "weight")
+        if self.stream not in ("model", "float32"):
+            raise ValueError(f"stream={self.stream!r}; choose 'model' or 'float32'")
+        if self.scale is not None and self.stream != "float32":
+            raise ValueError("a scaled embedding starts a 32-bit residual stream (stream='float32')")
         self.weight: torch.Tensor | None = None
 
     def param_infos(self):
-        return {"weight": ParamInfo((self.vocab, self.hidden))}
+        return {self.tensor: ParamInfo((self.vocab, self.hidden))}
 
     def load(self, tensors):
-        self.weight = tensors["weight"].contiguous()
+        self.weight = tensors[self.tensor].contiguous()
 
     def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
+        if self.stream == "float32":
+            out = torch.empty((token_ids.numel(), self.hidden), dtype=torch.float32, device=self.weight.device)
+            return ops.embed_scale(out, self.weight, token_ids, 1.0 if self.scale is None else float(self.scale))
         out = torch.empty((token_ids.numel(), self.hidden), dtype=self.weight.dtype, device=self.weight.device)
         return ops.embed_gather(out, self.weight, token_ids)
 
@@ -45,13 +57,14 @@ class LMHead(Part):
         self.vocab = int(spec["vocab"])
         self.hidden = int(spec["hidden"])
         self.tied = bool(spec.get("tied", False))
+        self.tensor = spec.get("tensor", "weight")  # the matrix's local name
         self.weight: torch.Tensor | None = None
 
     def param_infos(self):
-        return {} if self.tied else {"weight": ParamInfo((self.vocab, self.hidden))}
+        return {} if self.tied else {self.tensor: ParamInfo((self.vocab, self.hidden))}
 
     def load(self, tensors):
-        self.weight = tensors["weight"].contiguous()
+        self.weight = tensors["weight" if self.tied else self.tensor].contiguous()
 
     def forward(self, h) -> torch.Tensor:
         if isinstance(h, DeferredNorm):

@@ -11,8 +11,8 @@ from __future__ import annotations
 
 import torch
 
-from . import attention, block, embedding, rmsnorm, rope, swiglu  # noqa: F401  (register the built-in parts)
-from .registry import BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, BuildContext, DeferredNorm, Part
+from . import attention, attention_composed, block, embedding, gate, rmsnorm, rope, swiglu  # noqa: F401  (register the built-in parts)
+from .registry import BLOCKS, EMBEDDINGS, FEED_FORWARDS, GATES, HEADS, MIXERS, NORMS, BuildContext, DeferredNorm, Part
 from .spec import ModelSpec, ParamInfo
 
 
@@ -26,7 +26,7 @@ class Model:
         self.head = HEADS.build(spec.head, ctx)
         self.blocks = []
         self._sources = None
-        families = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS}
+        families = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS, "gate": GATES}
         for index, layer in enumerate(spec.layers):
             block = BLOCKS.get(layer.block)
             if set(layer.parts) != set(block.ROLES) or set(layer.weights) != set(block.ROLES):

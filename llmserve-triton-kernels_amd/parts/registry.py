@@ -178,11 +178,24 @@ class FeedForward(Part):
         raise NotImplementedError
 
 
+class Gate(Part):
+    """What a branch's result is multiplied by, element by element, before it joins the residual stream:
+    g = activation(products(h) + bias), h being the branch's own input.  `products` gives the 32-bit [N, hidden]
+    argument without the bias (None: the branch is not gated); an arrangement may stack the weights of its gates
+    (`weight`, [hidden, hidden]) into one product instead of calling it."""
+
+    weight = None
+    bias = None
+
+    def products(self, h: torch.Tensor):
+        return None
+
+
 class Block:
     """Arrangement of one layer's parts.
 
     `ROLES` maps every role of the arrangement to the family its part is built from ("mixer",
-    "feed_forward" or "norm"); the model builds a part for each role from the layer's spec and hands them
+    "feed_forward", "norm" or "gate"); the model builds a part for each role from the layer's spec and hands them
     over, and they are the block's attributes by role.  The part in the role "mixer", if the arrangement
     has one, is the one that keeps a cache between steps."""
 
@@ -232,6 +245,7 @@ POSITION_ENCODINGS = Registry("position encoding")
 MIXERS = Registry("mixer")
 FEED_FORWARDS = Registry("feed-forward")
 BLOCKS = Registry("block")
+GATES = Registry("gate")
 EMBEDDINGS = Registry("embedding")
 HEADS = Registry("output head")
 
@@ -240,3 +254,4 @@ register_position_encoding = POSITION_ENCODINGS.register
 register_mixer = MIXERS.register
 register_feed_forward = FEED_FORWARDS.register
 register_block = BLOCKS.register
+register_gate = GATES.register

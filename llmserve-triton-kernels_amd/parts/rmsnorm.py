@@ -46,3 +46,46 @@ class RMSNorm(Norm):
         if isinstance(delta, PartialSums):
             delta = delta.parts
         return ops.rmsnorm(out, x, self.weight, self.eps, delta=delta, rows=rows)
+
+
+@register_norm("rmsnorm32")
+class RMSNorm32(Norm):
+    """RMSNorm of a residual stream that is kept in 32-bit: x / sqrt(mean(x^2) + eps) * (offset + w), everything in
+    32-bit, rounded once to the model's dtype.  Parameters: hidden, eps, weight_offset (1.0 for a weight that is
+    stored as its deviation from one; default 0.0), tensor (the weight's local name; default "weight").  It offers
+    no `rms_params`: the products that norm their rows on the way in round where this norm does not."""
+
+    graph_safe = True
+
+    def __init__(self, spec, ctx):
+        super().__init__(spec, ctx)
+        self.hidden = int(spec["hidden"])
+        self.eps = float(spec["eps"])
+        self.offset = float(spec.get("weight_offset", 0.0))
+        self.tensor = spec.get("tensor", "weight")
+        self.weight: torch.Tensor | None = None
+
+    def param_infos(self):
+        return {self.tensor: ParamInfo((self.hidden,), "around_zero" if self.offset else "norm")}
+
+    def load(self, tensors):
+        self.weight = tensors[self.tensor].float().contiguous()
+
+    def forward(self, x):
+        out = torch.empty(x.shape, dtype=self.ctx.dtype, device=x.device)
+        return ops.rmsnorm32(out, self._stream(x), self.weight, self.eps, self.offset)
+
+    def add_norm(self, residual, delta):
+        if delta is not None:
+            raise ValueError("a 32-bit residual stream is summed by the arrangement, not by its norm")
+        return self.forward(residual)
+
+    def norm_rows(self, x, delta, rows):
+        if delta is not None:
+            raise ValueError("a 32-bit residual stream is summed by the arrangement, not by its norm")
+        out = torch.empty((rows.numel(), self.hidden), dtype=self.ctx.dtype, device=x.device)
+        return ops.rmsnorm32(out, self._stream(x), self.weight, self.eps, self.offset, rows=rows)
+
+    @staticmethod
+    def _stream(x):
+        return x if x.dtype == torch.float32 else x.float()

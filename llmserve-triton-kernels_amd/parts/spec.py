@@ -60,6 +60,7 @@ class ModelSpec:
     final_norm: PartSpec
     head: PartSpec
     weights: Mapping[str, str]  # roles "embedding", "final_norm", "head" -> checkpoint prefix
+    unused_tensors: tuple[str, ...] = ()  # names a checkpoint may hold without the model reading them
 
     def validate(self) -> None:
         n = len(self.layers)
@@ -92,11 +93,47 @@ class ModelSpec:
 
 @dataclass(frozen=True)
 class PagedCacheSpec:
-    """Keys and values of every token (or of the last `window` tokens) in pages."""
+    """Keys and values of every token in pages, or of those tokens a later query can still reach.
+
+    `window`: a query at position i reaches the keys j > i - window (None: no such limit).
+    `keep_first`: the keys j < keep_first stay reachable whatever the window.
+    `chunk`: a query reaches only keys of its own run of `chunk` positions, counted from position 0.
+    `value_heads`, `value_dim`: shape of the values where it differs from the keys' (None: the same)."""
 
     num_kv_heads: int
     head_dim: int
     window: int | None = None  # None: all keys are kept
+    keep_first: int = 0
+    chunk: int | None = None
+    value_heads: int | None = None
+    value_dim: int | None = None
+
+    @property
+    def v_heads(self) -> int:
+        return self.num_kv_heads if self.value_heads is None else self.value_heads
+
+    @property
+    def v_dim(self) -> int:
+        return self.head_dim if self.value_dim is None else self.value_dim
+
+    @property
+    def bounded(self) -> bool:
+        """Whether a request holds a bounded number of keys however long it grows."""
+        return self.window is not None or self.chunk is not None
+
+    def live_tokens(self) -> int:
+        """Most keys that queries from some position on can still reach, beside the kept first ones."""
+        spans = [n for n in (self.window, self.chunk) if n is not None]
+        return min(spans)
+
+    def dead_before(self, length: int) -> int:
+        """Keys at positions [keep_first, dead_before) are out of reach of every query at position >= length."""
+        dead = 0
+        if self.window is not None:
+            dead = max(dead, length - self.window + 1)
+        if self.chunk is not None:
+            dead = max(dead, length // self.chunk * self.chunk)
+        return dead
 
 
 @dataclass(frozen=True)

@@ -23,17 +23,22 @@ class SwiGLU(FeedForward):
         super().__init__(spec, ctx)
         self.hidden = int(spec["hidden"])
         self.intermediate = int(spec["intermediate"])
+        # `names`: local names of the three matrices; `result`: "float32" leaves the result unrounded for a caller
+        # that sums in 32-bit
+        names = spec.get("names") or {}
+        self.names = {k: names.get(k, f"{k}_proj.weight") for k in ("gate", "up", "down")}
+        self.result_dtype = torch.float32 if spec.get("result", "model") == "float32" else None
         self.gate_up: torch.Tensor | None = None
         self.down: torch.Tensor | None = None
 
     def param_infos(self):
         h, i = self.hidden, self.intermediate
-        return {"gate_proj.weight": ParamInfo((i, h)), "up_proj.weight": ParamInfo((i, h)),
-                "down_proj.weight": ParamInfo((h, i))}
+        return {self.names["gate"]: ParamInfo((i, h)), self.names["up"]: ParamInfo((i, h)),
+                self.names["down"]: ParamInfo((h, i))}
 
     def load(self, tensors):
-        self.gate_up = torch.cat([tensors["gate_proj.weight"], tensors["up_proj.weight"]], dim=0).contiguous()
-        self.down = tensors["down_proj.weight"].contiguous()
+        self.gate_up = torch.cat([tensors[self.names["gate"]], tensors[self.names["up"]]], dim=0).contiguous()
+        self.down = tensors[self.names["down"]].contiguous()
 
     def forward(self, x):
         deferred = isinstance(x, DeferredNorm)  # the caller hands the result to a norm, which takes partial sums
@@ -59,4 +64,15 @@ class SwiGLU(FeedForward):
         if deferred and x.may_add_in_place and adds_residual_in_epilogue(act, self.down):
             ops.gemm_decode(None, act, self.down, residual=x.residual)  # the residual sum in the product's epilogue
             return ADDED_IN_PLACE
-        return (linear_partial_sums(act, self.down) if deferred else None) or linear(act, self.down)
+        return (linear_partial_sums(act, self.down) if deferred else None) or linear(act, self.down,
+                                                                                       out_dtype=self.result_dtype)
+
+
+@register_feed_forward("none")
+class NoFeedForward(FeedForward):
+    """A layer without a feed-forward: nothing joins the stream."""
+
+    graph_safe = True
+
+    def forward(self, x):
+        return None

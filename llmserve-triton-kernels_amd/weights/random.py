@@ -46,6 +46,12 @@ def _fill_norm(shape, generator, device, options):
     return 1.0 + options["norm_std"] * torch.randn(shape, generator=generator, dtype=torch.float32, device=device)
 
 
+@register_initializer("around_zero")
+def _fill_around_zero(shape, generator, device, options):
+    """A weight stored as its deviation from one, a bias, a mixing vector: N(0, 10 norm_std)."""
+    return 10.0 * options["norm_std"] * torch.randn(shape, generator=generator, dtype=torch.float32, device=device)
+
+
 @register_initializer("zeros")
 def _fill_zeros(shape, generator, device, options):
     return torch.zeros(shape, dtype=torch.float32, device=device)
