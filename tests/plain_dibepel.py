@@ -66,6 +66,19 @@ def distance_slopes(heads: int) -> torch.Tensor:
     return torch.tensor([2.0 ** (-8.0 * (h + 1) / heads) for h in range(heads)], dtype=torch.float64)
 
 
+def differential_heads(q, k, v, visible, scale: float, lam: float, diff: float, eps: float) -> torch.Tensor:
+    """q [t, H, 2, dk], k [t, G, 2, dk], v [t, G, dv] -> [t, H, dv]: per head a_1 - lam a_2 over the same values,
+    divided by its root mean square, times (1 - diff)."""
+    t, H = q.shape[0], q.shape[1]
+    G = k.shape[1]
+    out = torch.zeros(t, H, v.shape[-1], dtype=q.dtype)
+    for head in range(H):
+        g = kv_head_of(head, H, G)
+        a = [masked_softmax((q[:, head, which] @ k[:, g, which].T) * scale, visible) @ v[:, g] for which in range(2)]
+        out[:, head] = rms_unit(a[0] - lam * a[1], eps) * (1.0 - diff)
+    return out
+
+
 def differential_attention(h: torch.Tensor, w: dict, p: str, m: dict, eps: float) -> torch.Tensor:
     """Two score maps per head over the same values; o = a1 - lambda a2, divided by its root mean square
     per head, times (1 - diff); then the output projection."""
@@ -78,16 +91,28 @@ def differential_attention(h: torch.Tensor, w: dict, p: str, m: dict, eps: float
     visible = visible_window(t, mask.get("size"), int(mask.get("keep_first") or 0))
     lam = (torch.exp((w[p + "lq1"] * w[p + "lk1"]).sum()) - torch.exp((w[p + "lq2"] * w[p + "lk2"]).sum())
            + m["diff"])
-    out = torch.zeros(t, H, dv, dtype=h.dtype)
-    for head in range(H):
-        g = kv_head_of(head, H, G)
-        a = []
-        for which in range(2):
-            s = (q[:, head, which] @ k[:, g, which].T) * m["scale"]
-            a.append(masked_softmax(s, visible) @ v[:, g])
-        o = a[0] - lam * a[1]
-        out[:, head] = rms_unit(o, eps) * (1.0 - m["diff"])
+    out = differential_heads(q, k, v, visible, m["scale"], lam, m["diff"], eps)
     return out.reshape(t, H * dv) @ w[p + "o"].T
+
+
+def talking_heads(q, k, v, visible, scale: float, slopes, talk) -> torch.Tensor:
+    """q [t, H, dk], k [t, G, dk], v [t, G, dv] -> [t, H, dv]: slope_h * (i - j) taken off the scores (slopes None:
+    nothing), softmax, the heads' weights mixed by `talk` (None: not mixed), each head on its own value head."""
+    t, H = q.shape[0], q.shape[1]
+    G = k.shape[1]
+    distance = (torch.arange(t)[:, None] - torch.arange(t)[None, :]).to(q.dtype)
+    weights = torch.zeros(H, t, t, dtype=q.dtype)
+    for head in range(H):
+        s = (q[:, head] @ k[:, kv_head_of(head, H, G)].T) * scale
+        if slopes is not None:
+            s = s - slopes[head] * distance
+        weights[head] = masked_softmax(s, visible)
+    if talk is not None:
+        weights = torch.einsum("hg,gij->hij", talk, weights)
+    out = torch.zeros(t, H, v.shape[-1], dtype=q.dtype)
+    for head in range(H):
+        out[:, head] = weights[head] @ v[:, kv_head_of(head, H, G)]
+    return out
 
 
 def talking_chunk_attention(h: torch.Tensor, w: dict, p: str, m: dict) -> torch.Tensor:
@@ -104,20 +129,8 @@ def talking_chunk_attention(h: torch.Tensor, w: dict, p: str, m: dict) -> torch.
     q = projected("q").view(t, H, dk)
     k = projected("k").view(t, G, dk)
     v = projected("v").view(t, G, dv)
-    visible = visible_chunk(t, mask.get("size"))
-    i = torch.arange(t)[:, None]
-    j = torch.arange(t)[None, :]
-    distance = (i - j).to(h.dtype)
-    slopes = distance_slopes(H).to(h.dtype)
-    weights = torch.zeros(H, t, t, dtype=h.dtype)
-    for head in range(H):
-        g = kv_head_of(head, H, G)
-        s = (q[:, head] @ k[:, g].T) * m["scale"] - slopes[head] * distance
-        weights[head] = masked_softmax(s, visible)
-    mixed = torch.einsum("hg,gij->hij", w[p + "talk"], weights)
-    out = torch.zeros(t, H, dv, dtype=h.dtype)
-    for head in range(H):
-        out[:, head] = mixed[head] @ v[:, kv_head_of(head, H, G)]
+    out = talking_heads(q, k, v, visible_chunk(t, mask.get("size")), m["scale"], distance_slopes(H).to(h.dtype),
+                        w[p + "talk"])
     return out.reshape(t, H * dv) @ w[p + "o"].T
 
 
@@ -161,3 +174,13 @@ def forward(config: dict, tensors: dict, ids: list[int], dtype=torch.float64, wi
 def lambda_of(w: dict, p: str, diff: float) -> float:
     return float(math.exp(float((w[p + "lq1"].double() * w[p + "lk1"].double()).sum()))
                  - math.exp(float((w[p + "lq2"].double() * w[p + "lk2"].double()).sum())) + diff)
+
+
+def greedy(config: dict, tensors: dict, prompt: list[int], n: int, dtype=torch.float64) -> list[int]:
+    """`n` tokens after `prompt`, each the argmax (lowest index wins) of a whole forward pass."""
+    ids, out = list(prompt), []
+    for _ in range(n):
+        tok = int(forward(config, tensors, ids, dtype)[-1].argmax())
+        out.append(tok)
+        ids.append(tok)
+    return out
