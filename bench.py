@@ -25,6 +25,13 @@ all arriving at once; `value` is generated tokens per second over the whole run,
 first token, inter-token latency percentiles and the number of preemptions beside it.
 `--pages-fraction` shrinks the cache pool below what the whole workload needs, so that
 requests wait and are preempted.
+
+    python bench.py --workload designs [--sizes 1b,7b] [--layers 6] [--batches 8,32] [--context 512]
+
+puts the Dibepel design beside the Llama decoder at equal layer sizes (width, heads, key/value heads, head size,
+feed-forward, vocabulary, layers; random weights): prefill tokens a second for one prompt of 2,048 tokens in one
+step, and decoded tokens a second at the given batch sizes behind `--context` tokens, both through the step
+function alone (no sampling); `value` is Dibepel's decode rate at the first size and batch.
 """
 
 from __future__ import annotations
@@ -181,6 +188,125 @@ def serve(args) -> int:
     return 0
 
 
+DESIGN_SIZES = {  # layer sizes of the named Llama shapes
+    "1b": dict(width=2048, ff=5632, heads=32, kv_heads=4, dim=64, vocab=32000),
+    "7b": dict(width=4096, ff=11008, heads=32, kv_heads=32, dim=128, vocab=32000),
+}
+
+
+def dibepel_config(size: dict, layers: int, window: int = 1024, keep_first: int = 64, chunk: int = 1024, taps: int = 4) -> dict:
+    """Every third layer the windowed attention with two score maps (half the heads, values twice as wide, so that
+    its projections have the sizes of the others'), the rest the chunked attention with convolutions and mixed heads."""
+    entries = []
+    for i in range(layers):
+        if i % 3 == 2:
+            mixer = {"heads": size["heads"] // 2, "kv_heads": max(1, size["kv_heads"] // 2), "dim": size["dim"],
+                     "vdim": 2 * size["dim"], "diff": 0.5, "scale": size["dim"] ** -0.5,
+                     "mask": {"size": window, "keep_first": keep_first}}
+            kind = "attention"
+        else:
+            mixer = {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["dim"], "vdim": size["dim"],
+                     "conv": taps, "scale": size["dim"] ** -0.5, "mask": {"size": chunk}}
+            kind = "attention_2"
+        entries.append({"type": kind, "mixer": mixer, "mlp": {"kind": "dense", "ff": size["ff"]}})
+    return {"architecture": "Dibepel", "vocab": size["vocab"], "width": size["width"], "embedding": {"scale": 1.0},
+            "norm": {"eps": 1e-5}, "layers": entries}
+
+
+def llama_config(size: dict, layers: int, positions: int) -> dict:
+    return dict(architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=size["vocab"], hidden_size=size["width"],
+                intermediate_size=size["ff"], num_hidden_layers=layers, num_attention_heads=size["heads"],
+                num_key_value_heads=size["kv_heads"], max_position_embeddings=positions, rope_theta=10000.0,
+                rms_norm_eps=1e-5)
+
+
+def designs(args) -> int:
+    """Dibepel beside the Llama decoder at equal sizes, through the step function alone."""
+    import torch
+
+    from llmserve import EngineConfig
+    from llmserve.engine.runner import ModelRunner, StepEntry
+
+    block_size = 16
+    batches = [int(b) for b in args.batches.split(",") if b]
+    steps, warmup = args.steps, args.warmup
+    longest = max(PREFILL_TOKENS, args.context + warmup + steps) + 8
+    pages = max(max(batches) * -(-(args.context + warmup + steps + 1) // block_size), -(-longest // block_size)) + 16
+    gen = torch.Generator().manual_seed(0)
+
+    def measure(config: dict) -> dict:
+        vocab = config.get("vocab") or config["vocab_size"]
+        engine_cfg = EngineConfig(dtype=args.dtype, block_size=block_size, num_blocks=pages, max_num_seqs=max(batches),
+                                  max_num_batched_tokens=PREFILL_TOKENS, max_model_len=longest)
+        runner = ModelRunner.from_random(config, seed=0, engine_config=engine_cfg)
+
+        def ids(n):
+            return torch.randint(0, vocab, (n,), generator=gen).tolist()
+
+        times = []
+        for _ in range(4):  # one prompt of 2,048 tokens in one step, the last token's logits wanted
+            runner.add_sequence("p")
+            tokens = ids(PREFILL_TOKENS)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            runner.step([StepEntry("p", tokens, [PREFILL_TOKENS - 1])])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+            runner.free_sequence("p")
+        pre_s = sorted(times[1:])[1]
+        out = {"prefill_tok_s": round(PREFILL_TOKENS / pre_s, 1), "prefill_ms": round(pre_s * 1e3, 3)}
+        for batch in batches:
+            names = [f"d{i}" for i in range(batch)]
+            for name in names:
+                runner.add_sequence(name)
+                left = args.context
+                while left > 0:  # the prompt in portions of the step budget
+                    n = min(left, PREFILL_TOKENS)
+                    runner.step([StepEntry(name, ids(n), [])])
+                    left -= n
+
+            def decode():
+                return runner.step([StepEntry(name, ids(1), [0]) for name in names], borrow=True)
+
+            for _ in range(warmup):
+                decode()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                decode()
+            torch.cuda.synchronize()
+            dt = (time.perf_counter() - t0) / steps
+            out[f"decode_b{batch}_tok_s"] = round(batch / dt, 1)
+            out[f"decode_b{batch}_ms"] = round(dt * 1e3, 4)
+            for name in names:
+                runner.free_sequence(name)
+        out["graphs"] = bool(runner._use_graphs)
+        del runner
+        torch.cuda.empty_cache()
+        return out
+
+    table = {}
+    for name in [s for s in args.sizes.split(",") if s]:
+        size = DESIGN_SIZES[name]
+        layers = args.layers or 6
+        row = {"layers": layers, **size, "dibepel": measure(dibepel_config(size, layers)),
+               "llama": measure(llama_config(size, layers, longest))}
+        row["dibepel_over_llama"] = {k: round(row["dibepel"][k] / row["llama"][k], 3) for k in row["dibepel"]
+                                     if k.endswith("tok_s")}
+        table[name] = row
+    first = table[next(iter(table))]
+    line = {"metric": "Dibepel beside Llama at equal layer sizes: decode tok/s (value: Dibepel, first size and batch), prefill tok/s",
+            "value": first["dibepel"][f"decode_b{batches[0]}_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": steps,
+            "warmup": warmup, "ms_per_step": first["dibepel"][f"decode_b{batches[0]}_ms"], "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+            "data": "synthetic", "config": {"model": "dibepel at llama layer sizes", "global_batch": batches[0],
+                                            "seq_len": args.context, "parallelism": "single-gpu", "weights": "random",
+                                            "prefill_tokens": PREFILL_TOKENS},
+            "designs": table}
+    print(json.dumps(line))
+    return 0
+
+
 def gemv(args) -> int:
     """The decode step's matrix products one by one, as the step's parts launch them (the kernel, the epilogue and
     the prologue they choose for the row count), at 1, 8, 32 and 64 rows.  Every launch of a chain takes the next of
@@ -299,7 +425,9 @@ def main() -> int:
     ap.add_argument("--phase", choices=["all", "decode", "prefill", "gemv"], default="all",
                     help="run one phase only (for profiles; the line then holds zeros for the other); gemv: the "
                          "decode products alone, each over copies of its weight that do not fit the caches")
-    ap.add_argument("--workload", choices=["steps", "serve"], default="steps")
+    ap.add_argument("--workload", choices=["steps", "serve", "designs"], default="steps")
+    ap.add_argument("--sizes", default="1b,7b", help="designs: layer sizes to compare at")
+    ap.add_argument("--batches", default="8,32", help="designs: decode batch sizes")
     ap.add_argument("--requests", type=int, default=64)
     ap.add_argument("--new-tokens", type=int, default=256)
     ap.add_argument("--prompt-min", type=int, default=128)
@@ -312,6 +440,8 @@ def main() -> int:
         return 2
     if args.workload == "serve":
         return serve(args)
+    if args.workload == "designs":
+        return designs(args)
     if args.phase == "gemv":
         return gemv(args)
 

@@ -1,0 +1,351 @@
+// The composed attention (see attention_composed.hip for its ingredients) on the matrix cores, bfloat16 storage.
+//
+// A *unit* is 16 columns that share a key/value head: `tpw` neighbouring tokens of one request times the `grp`
+// query heads of that key/value head (grp <= 16; columns beyond tpw * grp are padding).  A wave owns one or two
+// units.  Per tile of 16 keys it forms S^T = K Q^T with v_mfma_f32_16x16x16_bf16: the key rows are the A operand as
+// they lie in a page, the queries the B operand, and the result holds, per lane, 4 keys of one column, which is
+// exactly the B operand of O^T = V^T P^T; the values, transposed inside a page, are its A operand as they lie.
+// Scores, softmax, the mixing of heads and the difference of two maps are 32-bit; the weights are rounded to
+// bfloat16 only as the operand of the value product.
+//
+//   MAPS = 2   two score maps per query head over the same values, kept side by side in one wave (online
+//              softmax each), o = a_1 - lambda a_2, optionally normed per head.  A workgroup is 4 units of one
+//              key/value head; the grid runs over requests, blocks of tokens and key/value heads.
+//   TALK       the heads' normalised weights are mixed before they meet the values, so a workgroup holds every head
+//              of its tokens (up to 32 units in up to 16 waves) and walks the keys twice: once for every column's
+//              maximum and sum, once more to form the normalised weights, which go through LDS ([token][head][key],
+//              32-bit), are mixed per column by sum_g talk[h, g] w_g, and then multiply the values.
+//   neither    plain softmax attention with the same masks and slopes.
+//
+// Masks: a column at position i sees j <= i with j >= its chunk's start and (i - j < window or j < keep_first).
+// The tiles a workgroup walks are those its first token can reach up to its last token's position, and before
+// them the tiles of the kept first keys; what a column does not see is masked by comparison.  Keys of pages that
+// were given back (table entry < 0) and values behind the request's end are read as zeros.
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+struct MfmaArgs {
+    bf16* out;
+    const bf16* q;
+    const bf16* k_pool;
+    const bf16* v_pool;
+    const int* block_tables;
+    const int* table_rows;
+    const int* cu_seqlens;
+    const int* context_lens;
+    const float* slopes;
+    const float* talk;
+    int out_stride, q_stride, max_blocks;
+    int seq_begin, blocks_per_seq;
+    int heads, kv_heads, grp, dk, dv, block_size;
+    int window, keep_first, chunk;
+    int tok, tpw, upk, units, kv_per_wg;
+    float scale, lambda, eps, out_scale;
+    int head_norm;
+};
+
+__device__ __forceinline__ s16x4 load4(const bf16* p) { return *reinterpret_cast<const s16x4*>(p); }
+
+__device__ __forceinline__ s16x4 pack4(float a, float b, float c, float d) {
+    typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+    const u32x2 v = {pack_bf16x2(a, b), pack_bf16x2(c, d)};
+    return __builtin_bit_cast(s16x4, v);
+}
+
+__device__ __forceinline__ float column_max(float v) {  // over the 4 lanes that share a column
+    v = fmaxf(v, __shfl_xor(v, 16, LLMS_WAVE));
+    return fmaxf(v, __shfl_xor(v, 32, LLMS_WAVE));
+}
+
+__device__ __forceinline__ float column_sum(float v) {
+    v += __shfl_xor(v, 16, LLMS_WAVE);
+    return v + __shfl_xor(v, 32, LLMS_WAVE);
+}
+
+template <int MAPS, bool TALK, int MAXT, int MAXU, int THREADS>
+__global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) {
+    extern __shared__ float lds[];
+    const int wave = threadIdx.x / LLMS_WAVE, lane = threadIdx.x % LLMS_WAVE, nwaves = blockDim.x / LLMS_WAVE;
+    const int col = lane % 16, q4 = lane / 16;
+    const int b = a.seq_begin + blockIdx.x / a.blocks_per_seq, blk = blockIdx.x % a.blocks_per_seq;
+    const int row0 = a.cu_seqlens[b], count = a.cu_seqlens[b + 1] - row0;
+    const int end = a.context_lens[b];
+    const int t0 = blk * a.tok;
+    if (t0 >= count || end <= 0) return;  // (the same for every thread of the workgroup)
+    const int ntok = count - t0 < a.tok ? count - t0 : a.tok;
+    const int pos_lo = end - count + t0, pos_hi = pos_lo + ntok - 1;
+    const int* table = a.block_tables + (size_t)(a.table_rows ? a.table_rows[b] : b) * a.max_blocks;
+    const int kv_base = blockIdx.y * a.kv_per_wg;
+    const int H = a.heads, G = a.kv_heads, dk = a.dk, dv = a.dv, bs = a.block_size;
+    const int dkt = dk / 16, dvt = dv / 16;
+
+    // the tiles of 16 keys to walk: those of kept first keys that the first token's window has passed, then from
+    // the first key the first token reaches to the last token's own
+    const int lo_chunk = a.chunk > 0 ? pos_lo / a.chunk * a.chunk : 0;
+    const int lo_win = (a.window > 0 && pos_lo - a.window + 1 > 0) ? pos_lo - a.window + 1 : 0;
+    const int main_begin = (lo_chunk > lo_win ? lo_chunk : lo_win) / 16, main_end = pos_hi / 16 + 1;
+    int sink_begin = lo_chunk / 16, sink_end = (a.keep_first + 15) / 16;
+    if (sink_end > main_begin) sink_end = main_begin;
+    if (a.window <= 0 || sink_end < sink_begin) sink_end = sink_begin;
+    const int n_tiles = (sink_end - sink_begin) + (main_end - main_begin);
+
+    // this wave's units and columns
+    bool valid[MAXU];
+    int u_kvh[MAXU], u_h[MAXU], u_tl[MAXU], u_pos[MAXU], u_chunk_lo[MAXU];
+    float u_slope[MAXU];
+    s16x4 qf[MAXU][MAPS][MAXT];
+#pragma unroll
+    for (int uu = 0; uu < MAXU; ++uu) {
+        const int u = wave + uu * nwaves;
+        const bool active = u < a.units;
+        const int kvh = kv_base + (active ? u / a.upk : 0), sub = active ? u % a.upk : 0;
+        const int tl = sub * a.tpw + col / a.grp, h = kvh * a.grp + col % a.grp;
+        valid[uu] = active && col < a.tpw * a.grp && tl < ntok;
+        u_kvh[uu] = kvh, u_h[uu] = h, u_tl[uu] = tl, u_pos[uu] = pos_lo + tl;
+        u_chunk_lo[uu] = a.chunk > 0 ? u_pos[uu] / a.chunk * a.chunk : 0;
+        u_slope[uu] = (a.slopes && valid[uu]) ? a.slopes[h] : 0.f;
+        const bf16* qrow = a.q + (size_t)(row0 + t0 + tl) * a.q_stride + (size_t)h * MAPS * dk + 4 * q4;
+#pragma unroll
+        for (int m = 0; m < MAPS; ++m)
+#pragma unroll
+            for (int t = 0; t < MAXT; ++t)
+                qf[uu][m][t] = (valid[uu] && t < dkt) ? load4(qrow + m * dk + 16 * t) : s16x4{0, 0, 0, 0};
+    }
+
+    // scores of one tile for one unit and map: 4 keys (j0 + 4 q4 + r) of the lane's column, masked to -inf
+    auto scores = [&](int uu, int m, int j0, float sc[4]) {
+        const int j = j0 + col;  // the key whose row this lane brings
+        const int page = j <= pos_hi ? table[j / bs] : -1;
+        const bf16* krow = a.k_pool + (((size_t)(page < 0 ? 0 : page) * (G * MAPS) + u_kvh[uu] * MAPS + m) * bs + j % bs) * dk + 4 * q4;
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int t = 0; t < MAXT; ++t)
+            if (t < dkt) {
+                const s16x4 kf = page >= 0 ? load4(krow + 16 * t) : s16x4{0, 0, 0, 0};
+                acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kf, qf[uu][m][t], acc, 0, 0, 0);
+            }
+        const int pos = u_pos[uu];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int key = j0 + 4 * q4 + r;
+            const bool vis = valid[uu] && key <= pos && key >= u_chunk_lo[uu] &&
+                             (a.window <= 0 || pos - key < a.window || key < a.keep_first);
+            sc[r] = vis ? acc[r] * a.scale - u_slope[uu] * (float)(pos - key) : -INFINITY;
+        }
+    };
+    // O^T += V^T P^T for one unit: the values of key/value head u_kvh, keys j0 + 4 q4 .. + 3 of dimension 16 t + col
+    auto values = [&](int uu, int j0, s16x4 pf, f32x4 o[MAXT]) {
+        const int key = j0 + 4 * q4;
+        const int page = key < end ? table[key / bs] : -1;
+        const int keep = end - key;  // keys behind the request's end hold nothing
+        const bf16* vrow = a.v_pool + (((size_t)(page < 0 ? 0 : page) * G + u_kvh[uu]) * dv + col) * bs + key % bs;
+#pragma unroll
+        for (int t = 0; t < MAXT; ++t)
+            if (t < dvt) {
+                s16x4 vf = page >= 0 ? load4(vrow + (size_t)16 * t * bs) : s16x4{0, 0, 0, 0};
+                if (keep < 4) {
+                    if (keep < 2) vf.y = 0;
+                    if (keep < 3) vf.z = 0;
+                    vf.w = 0;
+                }
+                o[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pf, o[t], 0, 0, 0);
+            }
+    };
+    auto tile_start = [&](int i) { return 16 * (i < sink_end - sink_begin ? sink_begin + i : main_begin + i - (sink_end - sink_begin)); };
+
+    f32x4 acc_o[MAXU][MAPS][MAXT];
+    float run_m[MAXU][MAPS], run_l[MAXU][MAPS];
+#pragma unroll
+    for (int uu = 0; uu < MAXU; ++uu)
+#pragma unroll
+        for (int m = 0; m < MAPS; ++m) {
+            run_m[uu][m] = -INFINITY, run_l[uu][m] = 0.f;
+#pragma unroll
+            for (int t = 0; t < MAXT; ++t) acc_o[uu][m][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+
+    if constexpr (!TALK) {
+        for (int i = 0; i < n_tiles; ++i) {
+            const int j0 = tile_start(i);
+#pragma unroll
+            for (int uu = 0; uu < MAXU; ++uu) {
+                if (wave + uu * nwaves >= a.units) continue;
+#pragma unroll
+                for (int m = 0; m < MAPS; ++m) {
+                    float sc[4];
+                    scores(uu, m, j0, sc);
+                    const float m_new = fmaxf(run_m[uu][m], column_max(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]))));
+                    const float corr = m_new == -INFINITY ? 1.f : __expf(run_m[uu][m] - m_new);
+                    float p[4], sum = 0.f;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        p[r] = sc[r] == -INFINITY ? 0.f : __expf(sc[r] - m_new);
+                        sum += p[r];
+                    }
+                    run_l[uu][m] = run_l[uu][m] * corr + sum;
+                    run_m[uu][m] = m_new;
+#pragma unroll
+                    for (int t = 0; t < MAXT; ++t) acc_o[uu][m][t] *= corr;
+                    values(uu, j0, pack4(p[0], p[1], p[2], p[3]), acc_o[uu][m]);
+                }
+            }
+        }
+    } else {
+        float* pbuf = lds;                       // [tok][H][16]
+        float* talk_s = lds + a.tok * H * 16;     // [g][h]
+        for (int i = threadIdx.x; i < H * H; i += blockDim.x) talk_s[(i % H) * H + i / H] = a.talk[i];
+        // first walk: every column's maximum and sum
+        for (int i = 0; i < n_tiles; ++i) {
+            const int j0 = tile_start(i);
+#pragma unroll
+            for (int uu = 0; uu < MAXU; ++uu) {
+                if (wave + uu * nwaves >= a.units) continue;
+                float sc[4];
+                scores(uu, 0, j0, sc);
+                const float m_new = fmaxf(run_m[uu][0], column_max(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]))));
+                const float corr = m_new == -INFINITY ? 1.f : __expf(run_m[uu][0] - m_new);
+                float sum = 0.f;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) sum += sc[r] == -INFINITY ? 0.f : __expf(sc[r] - m_new);
+                run_l[uu][0] = run_l[uu][0] * corr + sum;
+                run_m[uu][0] = m_new;
+            }
+        }
+        float inv_l[MAXU];
+#pragma unroll
+        for (int uu = 0; uu < MAXU; ++uu) inv_l[uu] = 1.f / column_sum(run_l[uu][0]);
+        __syncthreads();  // (the mixing matrix is in LDS)
+        // second walk: normalised weights through LDS, mixed, times the values
+        for (int i = 0; i < n_tiles; ++i) {
+            const int j0 = tile_start(i);
+#pragma unroll
+            for (int uu = 0; uu < MAXU; ++uu) {
+                if (wave + uu * nwaves >= a.units) continue;
+                float sc[4];
+                scores(uu, 0, j0, sc);  // (every lane takes part: a padding column's lane still brings a key's row)
+                f32x4 w;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) w[r] = sc[r] == -INFINITY ? 0.f : __expf(sc[r] - run_m[uu][0]) * inv_l[uu];
+                if (col < a.tpw * a.grp) *reinterpret_cast<f32x4*>(pbuf + ((size_t)u_tl[uu] * H + u_h[uu]) * 16 + 4 * q4) = w;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int uu = 0; uu < MAXU; ++uu) {
+                if (wave + uu * nwaves >= a.units) continue;
+                f32x4 w = {0.f, 0.f, 0.f, 0.f};
+                if (col < a.tpw * a.grp) {
+                    const float* prow = pbuf + (size_t)u_tl[uu] * H * 16 + 4 * q4;
+                    const float* trow = talk_s + u_h[uu];
+                    for (int g = 0; g < H; ++g) {
+                        const f32x4 pg = *reinterpret_cast<const f32x4*>(prow + g * 16);
+                        const float tg = trow[g * H];
+                        w += tg * pg;
+                    }
+                }
+                values(uu, j0, pack4(w[0], w[1], w[2], w[3]), acc_o[uu][0]);
+            }
+            __syncthreads();
+        }
+    }
+
+    // what leaves: per column, 4 neighbouring dimensions per tile of 16
+#pragma unroll
+    for (int uu = 0; uu < MAXU; ++uu) {
+        if (wave + uu * nwaves >= a.units) continue;
+        float mul[MAPS];
+#pragma unroll
+        for (int m = 0; m < MAPS; ++m) mul[m] = TALK ? 1.f : 1.f / column_sum(run_l[uu][m]);
+        float ss = 0.f;
+#pragma unroll
+        for (int t = 0; t < MAXT; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float o = acc_o[uu][0][t][r] * mul[0];
+                if constexpr (MAPS == 2) o -= a.lambda * (acc_o[uu][1][t][r] * mul[1]);
+                acc_o[uu][0][t][r] = o;
+                if (t < dvt) ss = fmaf(o, o, ss);
+            }
+        float norm = 1.f;
+        if (a.head_norm) norm = a.out_scale / sqrtf(column_sum(ss) / (float)dv + a.eps);
+        if (!valid[uu]) continue;
+        bf16* orow = a.out + (size_t)(row0 + t0 + u_tl[uu]) * a.out_stride + (size_t)u_h[uu] * dv + 4 * q4;
+#pragma unroll
+        for (int t = 0; t < MAXT; ++t)
+            if (t < dvt) {
+                const f32x4 o = acc_o[uu][0][t] * norm;
+                *reinterpret_cast<s16x4*>(orow + 16 * t) = pack4(o[0], o[1], o[2], o[3]);
+            }
+    }
+}
+
+template <int MAPS, bool TALK, int MAXU, int THREADS>
+static int launch(const MfmaArgs& a, dim3 grid, int threads, size_t lds, hipStream_t stream) {
+    const int tiles = (a.dk > a.dv ? a.dk : a.dv) / 16;
+    if (tiles <= 4) {
+        auto kernel = attend_mfma_kernel<MAPS, TALK, 4, MAXU, THREADS>;
+        if (lds > 48 * 1024)
+            LLMS_HIP_CHECK(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        kernel<<<grid, threads, lds, stream>>>(a);
+    } else {
+        auto kernel = attend_mfma_kernel<MAPS, TALK, 8, MAXU, THREADS>;
+        if (lds > 48 * 1024)
+            LLMS_HIP_CHECK(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        kernel<<<grid, threads, lds, stream>>>(a);
+    }
+    LLMS_LAUNCH_CHECK();
+}
+
+extern "C" {
+
+// Rows [token rows of requests seq_begin .. seq_begin + n_seqs) of q and out; `max_new`: most tokens one of them brings.
+int llms_attend_composed_mfma(void* out, int out_stride, const void* q, int q_stride, const void* k_pool,
+                              const void* v_pool, const int* block_tables, const int* table_rows, int max_blocks,
+                              const int* cu_seqlens, const int* context_lens, int seq_begin, int n_seqs, int max_new,
+                              int heads, int kv_heads, int maps, int dk, int dv, int block_size, int window,
+                              int keep_first, int chunk, float scale, const float* slopes, const float* talk, float lambda,
+                              int head_norm, float eps, float out_scale, hipStream_t stream) {
+    LLMS_REQUIRE(n_seqs > 0 && max_new > 0 && heads > 0 && kv_heads > 0, "attend_composed_mfma: sizes must be positive");
+    LLMS_REQUIRE(heads % kv_heads == 0 && heads / kv_heads <= 16, "attend_composed_mfma: up to 16 query heads per key/value head");
+    LLMS_REQUIRE(maps == 1 || maps == 2, "attend_composed_mfma: one or two score maps");
+    LLMS_REQUIRE(!(talk && maps != 1), "attend_composed_mfma: mixing heads' weights goes with one score map");
+    LLMS_REQUIRE(dk % 16 == 0 && dv % 16 == 0 && dk <= 128 && dv <= 128 && dk > 0 && dv > 0,
+                 "attend_composed_mfma: key and value sizes are multiples of 16 up to 128");
+    LLMS_REQUIRE(block_size > 0 && block_size % 4 == 0 && max_blocks > 0, "attend_composed_mfma: pages of a multiple of 4 keys");
+    LLMS_REQUIRE(q_stride % 4 == 0 && out_stride % 4 == 0, "attend_composed_mfma: rows must be 8-byte aligned");
+    LLMS_REQUIRE(window >= 0 && keep_first >= 0 && chunk >= 0, "attend_composed_mfma: window, keep_first and chunk are >= 0");
+    MfmaArgs a;
+    a.out = (bf16*)out, a.q = (const bf16*)q, a.k_pool = (const bf16*)k_pool, a.v_pool = (const bf16*)v_pool;
+    a.block_tables = block_tables, a.table_rows = table_rows, a.cu_seqlens = cu_seqlens, a.context_lens = context_lens;
+    a.slopes = slopes, a.talk = talk;
+    a.out_stride = out_stride, a.q_stride = q_stride, a.max_blocks = max_blocks, a.seq_begin = seq_begin;
+    a.heads = heads, a.kv_heads = kv_heads, a.grp = heads / kv_heads, a.dk = dk, a.dv = dv, a.block_size = block_size;
+    a.window = window, a.keep_first = keep_first, a.chunk = chunk;
+    a.scale = scale, a.lambda = lambda, a.eps = eps, a.out_scale = out_scale, a.head_norm = head_norm;
+    a.tpw = 16 / a.grp;
+    if (talk) {
+        LLMS_REQUIRE(kv_heads <= 32, "attend_composed_mfma: mixing heads takes up to 32 key/value heads");
+        // every head of a block of tokens in one workgroup: up to 32 units in up to 16 waves
+        int upk = 32 / kv_heads;
+        while (upk > 1 && (upk - 1) * a.tpw >= max_new) --upk;  // (no more tokens than the longest portion has)
+        a.upk = upk, a.tok = upk * a.tpw, a.kv_per_wg = kv_heads, a.units = kv_heads * upk;
+        const int waves = a.units > 16 ? (a.units + 1) / 2 : a.units;
+        a.blocks_per_seq = (max_new + a.tok - 1) / a.tok;
+        const size_t lds = ((size_t)a.tok * heads * 16 + (size_t)heads * heads) * sizeof(float);
+        LLMS_REQUIRE(lds <= 160 * 1024, "attend_composed_mfma: too many heads for the LDS");
+        dim3 grid(n_seqs * a.blocks_per_seq, 1);
+        if (a.units > 16) return launch<1, true, 2, 1024>(a, grid, waves * LLMS_WAVE, lds, stream);
+        return launch<1, true, 1, 1024>(a, grid, waves * LLMS_WAVE, lds, stream);
+    }
+    int upk = 4;
+    while (upk > 1 && (upk - 1) * a.tpw >= max_new) --upk;
+    a.upk = upk, a.tok = upk * a.tpw, a.kv_per_wg = 1, a.units = upk;
+    a.blocks_per_seq = (max_new + a.tok - 1) / a.tok;
+    dim3 grid(n_seqs * a.blocks_per_seq, kv_heads);
+    LLMS_REQUIRE(grid.y <= 65535, "attend_composed_mfma: too many key/value heads");
+    if (maps == 2) return launch<2, false, 1, 256>(a, grid, upk * LLMS_WAVE, 0, stream);
+    return launch<1, false, 1, 256>(a, grid, upk * LLMS_WAVE, 0, stream);
+}
+
+}  // extern "C"

@@ -958,6 +958,74 @@ def attend_composed(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_
     return out
 
 
+def attend_composed_mfma_supported(dtype: torch.dtype, heads: int, kv_heads: int, dk: int, dv: int, block_size: int,
+                                    talk: bool) -> bool:
+    """Whether the matrix-core kernel takes this attention (else `attend_composed` does)."""
+    if dtype != torch.bfloat16 or heads % kv_heads or heads // kv_heads > 16:
+        return False
+    if dk % 16 or dv % 16 or not (0 < dk <= 128 and 0 < dv <= 128) or block_size % 4:
+        return False
+    if talk:
+        tok = max(1, 32 // kv_heads) * (16 // (heads // kv_heads))
+        return kv_heads <= 32 and (tok * heads * 16 + heads * heads) * 4 <= ATTEND_COMPOSED_LDS
+    return True
+
+
+def attend_composed_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                         block_tables: torch.Tensor, cu_seqlens: torch.Tensor, context_lens: torch.Tensor,
+                         seq_begin: int, n_seqs: int, max_new: int, *, heads: int, kv_heads: int, dk: int, dv: int,
+                         block_size: int, scale: float, maps: int = 1, window: int = 0, keep_first: int = 0,
+                         chunk: int = 0, slopes: torch.Tensor | None = None, talk: torch.Tensor | None = None,
+                         lam: float = 0.0, head_norm: bool = False, eps: float = 0.0, out_scale: float = 1.0,
+                         table_rows: torch.Tensor | None = None) -> torch.Tensor:
+    """`attend_composed` on the matrix cores (bfloat16) for requests [seq_begin, seq_begin + n_seqs) of a step: request
+    b owns rows cu_seqlens[b] .. cu_seqlens[b+1] of q and out, brings at most `max_new` tokens and is context_lens[b]
+    long after the step (0: padding, left alone).  Same arguments and arithmetic otherwise; the weights are rounded
+    to bfloat16 as the operand of the value product."""
+    dev = _dev(out, q, k_pool, v_pool, block_tables, cu_seqlens, context_lens, slopes, talk, table_rows)
+    if not attend_composed_mfma_supported(q.dtype, heads, kv_heads, dk, dv, block_size, talk is not None):
+        raise ValueError("attend_composed_mfma does not take these sizes; see attend_composed_mfma_supported")
+    if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < heads * maps * dk or q.stride(0) % 4 or q.data_ptr() % 8:
+        raise ValueError("q must be [N, >= heads*maps*dk] with unit inner stride and 8-byte aligned rows")
+    _rows(out, "out", heads * dv)
+    if out.shape[0] != q.shape[0] or out.dtype != q.dtype or out.data_ptr() % 8:
+        raise ValueError("out and q disagree")
+    pages = k_pool.shape[0]
+    if tuple(k_pool.shape) != (pages, kv_heads * maps, block_size, dk) or not k_pool.is_contiguous():
+        raise ValueError(f"k_pool shape {tuple(k_pool.shape)} is not [pages,{kv_heads * maps},{block_size},{dk}]")
+    if tuple(v_pool.shape) != (pages, kv_heads, dv, block_size) or not v_pool.is_contiguous():
+        raise ValueError(f"v_pool shape {tuple(v_pool.shape)} is not [pages,{kv_heads},{dv},{block_size}]")
+    if k_pool.dtype != q.dtype or v_pool.dtype != q.dtype or k_pool.data_ptr() % 8 or v_pool.data_ptr() % 8:
+        raise ValueError("pools and q differ in dtype, or a pool is not 8-byte aligned")
+    if block_tables.dim() != 2 or block_tables.dtype != torch.int32 or not block_tables.is_contiguous():
+        raise ValueError("block_tables must be a contiguous int32 [B, M] tensor")
+    if maps not in (1, 2) or (talk is not None and maps != 1):
+        raise ValueError("maps is 1 or 2, and talk goes with maps = 1")
+    _i32(cu_seqlens, "cu_seqlens")
+    b = cu_seqlens.numel() - 1
+    _i32(context_lens, "context_lens", b)
+    if table_rows is not None:
+        _i32(table_rows, "table_rows", b)
+    elif block_tables.shape[0] < b:
+        raise ValueError("block_tables has fewer rows than there are requests")
+    if not (0 <= seq_begin and n_seqs >= 0 and seq_begin + n_seqs <= b):
+        raise ValueError("request range is outside the batch")
+    if slopes is not None:
+        _f32(slopes, "slopes", heads)
+    if talk is not None:
+        _f32(talk, "talk", heads * heads)
+    if n_seqs == 0 or max_new <= 0 or q.shape[0] == 0:
+        return out
+    _check(load("attention_composed_mfma").llms_attend_composed_mfma(
+        _ptr(out), c_int(out.stride(0)), _ptr(q), c_int(q.stride(0)), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables),
+        _ptr(table_rows), c_int(block_tables.shape[1]), _ptr(cu_seqlens), _ptr(context_lens), c_int(seq_begin),
+        c_int(n_seqs), c_int(max_new), c_int(heads), c_int(kv_heads), c_int(maps), c_int(dk), c_int(dv),
+        c_int(block_size), c_int(window), c_int(keep_first), c_int(chunk), c_float(scale), _ptr(slopes), _ptr(talk),
+        c_float(lam), c_int(1 if head_norm else 0), c_float(eps), c_float(out_scale), _stream(dev)),
+        "attend_composed_mfma")
+    return out
+
+
 # ------------------------------------------------------------------------------ sampling
 
 

@@ -155,11 +155,26 @@ class ComposedAttention(Mixer):
         if conv:
             ops.conv_state(state.state, proj, batch.state_slots, batch.cu_seqlens, batch.context_lens)
         out = torch.empty((proj.shape[0], heads * dv), dtype=x.dtype, device=x.device)
-        ops.attend_composed(out, q, paged.k_pool, paged.v_pool, view.block_tables, batch.token_seq, batch.positions,
-                            heads=heads, kv_heads=kv, dk=dk, dv=dv, block_size=paged.block_size, scale=self.scale,
-                            maps=self.maps, window=int(self.window or 0), keep_first=self.keep_first,
-                            chunk=int(self.chunk or 0), slopes=self.slopes, talk=self.talk, lam=self.lam,
-                            head_norm=self.head_norm_eps is not None, eps=float(self.head_norm_eps or 0.0),
-                            out_scale=self.head_norm_scale, table_rows=batch.state_slots,
-                            context_lens=batch.context_lens)
+        self.attend(out, q, paged, view, batch)
         return linear(out, self.o_weight, out_dtype=self.result_dtype)
+
+    def attend(self, out, q, paged, view, batch):
+        """out[n] = this attention of token n's heads over its request's pages: on the matrix cores where the
+        sizes allow (bfloat16; requests that bring one token in one launch, portions of prompts in another), else
+        by the kernel that takes any size and dtype."""
+        common = dict(heads=self.num_heads, kv_heads=self.num_kv_heads, dk=self.head_dim, dv=self.value_dim,
+                      block_size=paged.block_size, scale=self.scale, maps=self.maps, window=int(self.window or 0),
+                      keep_first=self.keep_first, chunk=int(self.chunk or 0), slopes=self.slopes, talk=self.talk,
+                      lam=self.lam, head_norm=self.head_norm_eps is not None, eps=float(self.head_norm_eps or 0.0),
+                      out_scale=self.head_norm_scale, table_rows=batch.state_slots)
+        if not ops.attend_composed_mfma_supported(q.dtype, self.num_heads, self.num_kv_heads, self.head_dim,
+                                                  self.value_dim, paged.block_size, self.talking):
+            ops.attend_composed(out, q, paged.k_pool, paged.v_pool, view.block_tables, batch.token_seq, batch.positions,
+                                context_lens=batch.context_lens, **common)
+            return
+        args = (out, q, paged.k_pool, paged.v_pool, view.block_tables, batch.cu_seqlens, batch.context_lens)
+        n_dec = batch.num_decode
+        if n_dec:
+            ops.attend_composed_mfma(*args, 0, n_dec, 1, **common)
+        if n_dec < batch.num_seqs:
+            ops.attend_composed_mfma(*args, n_dec, batch.num_seqs - n_dec, batch.max_count, **common)

@@ -53,3 +53,14 @@ SMALL_B = config_of(width=64, vocab=97, scale=1.0, eps=1e-6, ff=40, layers=[
     ("attention_2", {"weights_of": 1}),
     ("attention_2", {"mixer": {"heads": 5, "kv_heads": 5, "dim": 12, "vdim": 20, "conv": 4, "mask": {"size": 3}}}),
 ])
+
+# sizes the matrix-core attention takes (keys and values in multiples of 16), with 1, 2 and 8 query heads per
+# key/value head
+SMALL_C = config_of(width=64, vocab=131, scale=0.8, ff=48, layers=[
+    ("attention_2", {"mixer": {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 32, "conv": 3, "mask": {"size": 20}}}),
+    ("attention", {"mixer": {"heads": 2, "kv_heads": 1, "dim": 32, "vdim": 16, "mask": {"size": 11, "keep_first": 6}}}),
+    ("attention_2", {"mixer": {"heads": 8, "kv_heads": 1, "dim": 16, "vdim": 16, "conv": 2, "mask": {"size": 64}}}),
+    ("attention", {"weights_of": 1}),
+    ("attention_2", {"mixer": {"heads": 3, "kv_heads": 3, "dim": 16, "vdim": 16, "conv": 1, "mask": {"size": 9}}}),
+    ("attention", {"mixer": {"heads": 4, "kv_heads": 4, "dim": 16, "vdim": 48, "diff": 0.1, "mask": {"size": 40, "keep_first": 20}}}),
+])

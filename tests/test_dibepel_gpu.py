@@ -9,7 +9,7 @@ import torch
 
 import plain_dibepel as pd
 import traces
-from dibepel_configs import SMALL, SMALL_B, config_of
+from dibepel_configs import SMALL, SMALL_B, SMALL_C, config_of
 
 pytestmark = pytest.mark.gpu
 
@@ -249,6 +249,97 @@ def test_a_key_that_stands_out_shows_every_edge():
     assert not marker_seen(299, 99, slopes=slope) and marker_seen(299, 290, slopes=slope)
 
 
+# ------------------------------------------------------------------------------ the matrix-core kernel
+def attend_mfma(seqs, bs, **kw):
+    """`seqs`: per request (q [t, S, dk], k, v, first new row, number of new rows); requests that bring one row
+    first.  All share one pool.  Returns the kernel's rows per request."""
+    from llmserve.ops import library as ops
+
+    dt = torch.bfloat16
+    pools = [paged(k, v, bs, dt, seed=i) for i, (_q, k, v, _a, _n) in enumerate(seqs)]
+    k_pool = torch.cat([p[0] for p in pools])
+    v_pool = torch.cat([p[1] for p in pools])
+    width = max(p[2].shape[1] for p in pools)
+    table = torch.zeros((len(seqs) + 2, width), dtype=torch.int32, device=DEV)
+    rows_of = [len(seqs) + 1 - i for i in range(len(seqs))]  # (a request's row of the table is not its index)
+    base = 0
+    for i, p in enumerate(pools):
+        table[rows_of[i], : p[2].shape[1]] = p[2][0] + base
+        base += p[0].shape[0]
+    qs = torch.cat([q[a: a + n].reshape(n, -1) for q, _k, _v, a, n in seqs]).to(dt).to(DEV)
+    cu = [0]
+    for *_x, n in seqs:
+        cu.append(cu[-1] + n)
+    as_i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)  # noqa: E731
+    heads, dv = kw["heads"], seqs[0][2].shape[2]
+    out = torch.full((qs.shape[0], heads * dv), float("nan"), dtype=dt, device=DEV)
+    n_dec = sum(1 for *_x, n in seqs if n == 1)
+    args = (out, qs, k_pool, v_pool, table, as_i32(cu), as_i32([a + n for *_x, a, n in seqs]))
+    common = dict(dk=seqs[0][0].shape[2], dv=dv, block_size=bs, table_rows=as_i32(rows_of), **kw)
+    if n_dec:
+        ops.attend_composed_mfma(*args, 0, n_dec, 1, **common)
+    if n_dec < len(seqs):
+        ops.attend_composed_mfma(*args, n_dec, len(seqs) - n_dec, max(n for *_x, n in seqs), **common)
+    return [out[cu[i]: cu[i + 1]] for i in range(len(seqs))]
+
+
+MFMA_DIFF = [  # heads, kv_heads, dk, dv, window, keep_first, block size
+    (2, 1, 32, 16, 11, 6, 8),
+    (4, 4, 16, 48, 40, 20, 16),
+    (16, 2, 64, 128, 33, 0, 16),
+    (3, 1, 16, 16, None, 0, 4),  # three heads in a unit of 16 columns: five tokens and a padded column
+]
+
+
+@pytest.mark.parametrize("heads,kv,dk,dv,window,keep,bs", MFMA_DIFF)
+def test_matrix_core_kernel_two_maps(heads, kv, dk, dv, window, keep, bs):
+    dt = torch.bfloat16
+    lam, diff, eps, scale = 0.83, 0.3, 1e-5, 0.3
+    seqs, refs = [], []
+    for i, (t, first, n) in enumerate([(71, 70, 1), (150, 149, 1), (90, 0, 90), (58, 33, 25), (40, 38, 2)]):
+        q, k, v = (rounded(x, dt) for x in (rnd(t, heads, 2, dk, seed=60 + i), rnd(t, kv, 2, dk, seed=70 + i),
+                                            rnd(t, kv, dv, seed=80 + i)))
+        ref = pd.differential_heads(q, k, v, pd.visible_window(t, window, keep), scale, lam, diff, eps)
+        refs.append(ref.reshape(t, -1)[first: first + n])
+        seqs.append((q.reshape(t, heads * 2, dk), k.reshape(t, kv * 2, dk), v, first, n))
+    got = attend_mfma(seqs, bs, heads=heads, kv_heads=kv, maps=2, window=window or 0, keep_first=keep, scale=scale,
+                      lam=lam, head_norm=True, eps=eps, out_scale=1 - diff)
+    for i, (g, r) in enumerate(zip(got, refs)):
+        close(g, r, dt, f"request {i}")
+
+
+MFMA_TALK = [  # heads, kv_heads, dk, dv, chunk, block size
+    (4, 2, 16, 32, 20, 8),
+    (8, 1, 16, 16, 64, 16),
+    (3, 3, 16, 16, 9, 8),
+    (32, 4, 64, 64, 128, 16),
+    (32, 32, 32, 128, None, 16),  # two units a wave
+    (6, 2, 16, 16, 50, 4),
+]
+
+
+@pytest.mark.parametrize("heads,kv,dk,dv,chunk,bs", MFMA_TALK)
+def test_matrix_core_kernel_mixed_heads(heads, kv, dk, dv, chunk, bs):
+    dt = torch.bfloat16
+    talk = torch.eye(heads, dtype=F64) + rnd(heads, heads, seed=33, scale=0.3 / heads ** 0.5)
+    slopes = pd.distance_slopes(heads)
+    seqs, refs = [], []
+    for i, (t, first, n) in enumerate([(71, 70, 1), (130, 129, 1), (90, 0, 90), (58, 33, 25), (40, 38, 2)]):
+        q, k, v = (rounded(x, dt) for x in (rnd(t, heads, dk, seed=60 + i), rnd(t, kv, dk, seed=70 + i),
+                                            rnd(t, kv, dv, seed=80 + i)))
+        ref = pd.talking_heads(q, k, v, pd.visible_chunk(t, chunk), 0.3, slopes, talk)
+        refs.append(ref.reshape(t, -1)[first: first + n])
+        seqs.append((q, k, v, first, n))
+    got = attend_mfma(seqs, bs, heads=heads, kv_heads=kv, chunk=chunk or 0, scale=0.3, slopes=slopes.float().to(DEV),
+                      talk=talk.float().to(DEV))
+    for i, (g, r) in enumerate(zip(got, refs)):
+        close(g, r, dt, f"request {i}")
+    got = attend_mfma(seqs[2:3], bs, heads=heads, kv_heads=kv, chunk=chunk or 0, scale=0.3)  # neither slopes nor mixing
+    ref = pd.talking_heads(seqs[2][0].double(), seqs[2][1].double(), seqs[2][2].double(), pd.visible_chunk(90, chunk), 0.3,
+                           None, None)
+    close(got[0], ref.reshape(90, -1), dt, "plain")
+
+
 # ------------------------------------------------------------------------------ whole models
 def write_model(folder, config, seed):
     from safetensors.torch import load_file
@@ -273,7 +364,7 @@ def logits_close(got, ref, dtype, what):
     assert float(err.max()) <= limit, f"{what}: position {worst} is off by {float(err.max()):.2e} (limit {limit})"
 
 
-MODELS = {"small": (SMALL, 8), "small_b": (SMALL_B, 16)}
+MODELS = {"small": (SMALL, 8), "small_b": (SMALL_B, 16), "small_c": (SMALL_C, 8)}
 
 
 @pytest.fixture(scope="module")
