@@ -17,6 +17,12 @@
 //              32-bit), are mixed per column by sum_g talk[h, g] w_g, and then multiply the values.
 //   neither    plain softmax attention with the same masks and slopes.
 //
+// Keys are walked in groups of TG tiles: all of a group's key rows are asked for before the first product, all its
+// values before the softmax arithmetic, so a wave waits for memory once per 16 TG keys.  When a workgroup holds no
+// more tokens than one unit (decoding), the groups are dealt to `slices` waves per unit, which merge through LDS at
+// the end (maxima, sums and partial results; with TALK the maxima and sums after the first walk, the partial
+// results, already normalised, after the second).
+//
 // Masks: a column at position i sees j <= i with j >= its chunk's start and (i - j < window or j < keep_first).
 // The tiles a workgroup walks are those its first token can reach up to its last token's position, and before
 // them the tiles of the kept first keys; what a column does not see is masked by comparison.  Keys of pages that
@@ -41,7 +47,7 @@ struct MfmaArgs {
     int seq_begin, blocks_per_seq;
     int heads, kv_heads, grp, dk, dv, block_size;
     int window, keep_first, chunk;
-    int tok, tpw, upk, units, kv_per_wg;
+    int tok, tpw, upk, units, kv_per_wg, slices;
     float scale, lambda, eps, out_scale;
     int head_norm;
 };
@@ -64,11 +70,12 @@ __device__ __forceinline__ float column_sum(float v) {
     return v + __shfl_xor(v, 32, LLMS_WAVE);
 }
 
-template <int MAPS, bool TALK, int MAXT, int MAXU, int THREADS>
+template <int MAPS, bool TALK, int MAXTK, int MAXTV, int MAXU, int TG, int THREADS>
 __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) {
     extern __shared__ float lds[];
     const int wave = threadIdx.x / LLMS_WAVE, lane = threadIdx.x % LLMS_WAVE, nwaves = blockDim.x / LLMS_WAVE;
     const int col = lane % 16, q4 = lane / 16;
+    const int NS = a.slices, slice = wave % NS, uw = wave / NS, n_uw = nwaves / NS;
     const int b = a.seq_begin + blockIdx.x / a.blocks_per_seq, blk = blockIdx.x % a.blocks_per_seq;
     const int row0 = a.cu_seqlens[b], count = a.cu_seqlens[b + 1] - row0;
     const int end = a.context_lens[b];
@@ -80,6 +87,7 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
     const int kv_base = blockIdx.y * a.kv_per_wg;
     const int H = a.heads, G = a.kv_heads, dk = a.dk, dv = a.dv, bs = a.block_size;
     const int dkt = dk / 16, dvt = dv / 16;
+    const int used_cols = a.tpw * a.grp;
 
     // the tiles of 16 keys to walk: those of kept first keys that the first token's window has passed, then from
     // the first key the first token reaches to the last token's own
@@ -89,20 +97,25 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
     int sink_begin = lo_chunk / 16, sink_end = (a.keep_first + 15) / 16;
     if (sink_end > main_begin) sink_end = main_begin;
     if (a.window <= 0 || sink_end < sink_begin) sink_end = sink_begin;
-    const int n_tiles = (sink_end - sink_begin) + (main_end - main_begin);
+    const int n_sink = sink_end - sink_begin;
+    const int n_tiles = n_sink + (main_end - main_begin);
+    const int n_groups = (n_tiles + TG - 1) / TG;
+    const int n_rounds = (n_groups + NS - 1) / NS;  // every slice walks this many groups (the last may be empty)
+    // first key of tile i; tiles behind the last lie behind every token's position and hold nothing
+    auto tile_start = [&](int i) { return 16 * (i < n_sink ? sink_begin + i : main_begin + (i - n_sink)); };
 
     // this wave's units and columns
-    bool valid[MAXU];
+    bool valid[MAXU], mine[MAXU];
     int u_kvh[MAXU], u_h[MAXU], u_tl[MAXU], u_pos[MAXU], u_chunk_lo[MAXU];
     float u_slope[MAXU];
-    s16x4 qf[MAXU][MAPS][MAXT];
+    s16x4 qf[MAXU][MAPS][MAXTK];
 #pragma unroll
     for (int uu = 0; uu < MAXU; ++uu) {
-        const int u = wave + uu * nwaves;
-        const bool active = u < a.units;
-        const int kvh = kv_base + (active ? u / a.upk : 0), sub = active ? u % a.upk : 0;
+        const int u = uw + uu * n_uw;
+        mine[uu] = u < a.units;
+        const int kvh = kv_base + (mine[uu] ? u / a.upk : 0), sub = mine[uu] ? u % a.upk : 0;
         const int tl = sub * a.tpw + col / a.grp, h = kvh * a.grp + col % a.grp;
-        valid[uu] = active && col < a.tpw * a.grp && tl < ntok;
+        valid[uu] = mine[uu] && col < used_cols && tl < ntok;
         u_kvh[uu] = kvh, u_h[uu] = h, u_tl[uu] = tl, u_pos[uu] = pos_lo + tl;
         u_chunk_lo[uu] = a.chunk > 0 ? u_pos[uu] / a.chunk * a.chunk : 0;
         u_slope[uu] = (a.slopes && valid[uu]) ? a.slopes[h] : 0.f;
@@ -110,156 +123,290 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
 #pragma unroll
         for (int m = 0; m < MAPS; ++m)
 #pragma unroll
-            for (int t = 0; t < MAXT; ++t)
+            for (int t = 0; t < MAXTK; ++t)
                 qf[uu][m][t] = (valid[uu] && t < dkt) ? load4(qrow + m * dk + 16 * t) : s16x4{0, 0, 0, 0};
     }
 
-    // scores of one tile for one unit and map: 4 keys (j0 + 4 q4 + r) of the lane's column, masked to -inf
-    auto scores = [&](int uu, int m, int j0, float sc[4]) {
-        const int j = j0 + col;  // the key whose row this lane brings
-        const int page = j <= pos_hi ? table[j / bs] : -1;
-        const bf16* krow = a.k_pool + (((size_t)(page < 0 ? 0 : page) * (G * MAPS) + u_kvh[uu] * MAPS + m) * bs + j % bs) * dk + 4 * q4;
-        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    // scores of one group of tiles for one unit and map: per tile 4 keys (j0 + 4 q4 + r) of the lane's column,
+    // masked to -inf.  Every lane takes part, also one whose column is padding: it still brings a key's row.
+    auto scores = [&](int uu, int m, int group, float sc[TG][4]) {
+        s16x4 kf[TG][MAXTK];
 #pragma unroll
-        for (int t = 0; t < MAXT; ++t)
-            if (t < dkt) {
-                const s16x4 kf = page >= 0 ? load4(krow + 16 * t) : s16x4{0, 0, 0, 0};
-                acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kf, qf[uu][m][t], acc, 0, 0, 0);
-            }
+        for (int tt = 0; tt < TG; ++tt) {
+            const int j = tile_start(group * TG + tt) + col;  // the key whose row this lane brings
+            const int page = j <= pos_hi ? table[j / bs] : -1;
+            const bf16* krow = a.k_pool + (((size_t)(page < 0 ? 0 : page) * (G * MAPS) + u_kvh[uu] * MAPS + m) * bs + j % bs) * dk + 4 * q4;
+#pragma unroll
+            for (int t = 0; t < MAXTK; ++t) kf[tt][t] = (page >= 0 && t < dkt) ? load4(krow + 16 * t) : s16x4{0, 0, 0, 0};
+        }
         const int pos = u_pos[uu];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int key = j0 + 4 * q4 + r;
-            const bool vis = valid[uu] && key <= pos && key >= u_chunk_lo[uu] &&
-                             (a.window <= 0 || pos - key < a.window || key < a.keep_first);
-            sc[r] = vis ? acc[r] * a.scale - u_slope[uu] * (float)(pos - key) : -INFINITY;
+        for (int tt = 0; tt < TG; ++tt) {
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int t = 0; t < MAXTK; ++t)
+                if (t < dkt) acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kf[tt][t], qf[uu][m][t], acc, 0, 0, 0);
+            const int j0 = tile_start(group * TG + tt);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int key = j0 + 4 * q4 + r;
+                const bool vis = valid[uu] && key <= pos && key >= u_chunk_lo[uu] &&
+                                 (a.window <= 0 || pos - key < a.window || key < a.keep_first);
+                sc[tt][r] = vis ? acc[r] * a.scale - u_slope[uu] * (float)(pos - key) : -INFINITY;
+            }
         }
     };
-    // O^T += V^T P^T for one unit: the values of key/value head u_kvh, keys j0 + 4 q4 .. + 3 of dimension 16 t + col
-    auto values = [&](int uu, int j0, s16x4 pf, f32x4 o[MAXT]) {
-        const int key = j0 + 4 * q4;
-        const int page = key < end ? table[key / bs] : -1;
-        const int keep = end - key;  // keys behind the request's end hold nothing
-        const bf16* vrow = a.v_pool + (((size_t)(page < 0 ? 0 : page) * G + u_kvh[uu]) * dv + col) * bs + key % bs;
+    // the values of key/value head u_kvh for one group: per tile, keys j0 + 4 q4 .. + 3 of dimension 16 t + col
+    auto load_values = [&](int uu, int group, s16x4 vf[TG][MAXTV]) {
 #pragma unroll
-        for (int t = 0; t < MAXT; ++t)
-            if (t < dvt) {
-                s16x4 vf = page >= 0 ? load4(vrow + (size_t)16 * t * bs) : s16x4{0, 0, 0, 0};
+        for (int tt = 0; tt < TG; ++tt) {
+            const int key = tile_start(group * TG + tt) + 4 * q4;
+            const int page = key < end ? table[key / bs] : -1;
+            const int keep = end - key;  // keys behind the request's end hold nothing
+            const bf16* vrow = a.v_pool + (((size_t)(page < 0 ? 0 : page) * G + u_kvh[uu]) * dv + col) * bs + key % bs;
+#pragma unroll
+            for (int t = 0; t < MAXTV; ++t) {
+                s16x4 v = (page >= 0 && t < dvt) ? load4(vrow + (size_t)16 * t * bs) : s16x4{0, 0, 0, 0};
                 if (keep < 4) {
-                    if (keep < 2) vf.y = 0;
-                    if (keep < 3) vf.z = 0;
-                    vf.w = 0;
+                    if (keep < 2) v.y = 0;
+                    if (keep < 3) v.z = 0;
+                    v.w = 0;
                 }
-                o[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pf, o[t], 0, 0, 0);
+                vf[tt][t] = v;
             }
+        }
     };
-    auto tile_start = [&](int i) { return 16 * (i < sink_end - sink_begin ? sink_begin + i : main_begin + i - (sink_end - sink_begin)); };
+    auto times_values = [&](const s16x4 vf[TG][MAXTV], const s16x4 pf[TG], f32x4 o[MAXTV]) {
+#pragma unroll
+        for (int tt = 0; tt < TG; ++tt)
+#pragma unroll
+            for (int t = 0; t < MAXTV; ++t)
+                if (t < dvt) o[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf[tt][t], pf[tt], o[t], 0, 0, 0);
+    };
 
-    f32x4 acc_o[MAXU][MAPS][MAXT];
-    float run_m[MAXU][MAPS], run_l[MAXU][MAPS];
+    f32x4 acc_o[MAXU][MAPS][MAXTV];
+    float run_m[MAXU][MAPS], run_l[MAXU][MAPS];  // (a lane's share of its column's sum)
 #pragma unroll
     for (int uu = 0; uu < MAXU; ++uu)
 #pragma unroll
         for (int m = 0; m < MAPS; ++m) {
             run_m[uu][m] = -INFINITY, run_l[uu][m] = 0.f;
 #pragma unroll
-            for (int t = 0; t < MAXT; ++t) acc_o[uu][m][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int t = 0; t < MAXTV; ++t) acc_o[uu][m][t] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
+    // a group's scores join a column's running maximum and sum; returns the factor for what was gathered before
+    auto join = [&](const float sc[TG][4], float& m_run, float& l_run, float p[TG][4]) {
+        float mx = -INFINITY;
+#pragma unroll
+        for (int tt = 0; tt < TG; ++tt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) mx = fmaxf(mx, sc[tt][r]);
+        const float m_new = fmaxf(m_run, column_max(mx));
+        const float corr = m_new == -INFINITY ? 1.f : __expf(m_run - m_new);
+        float sum = 0.f;
+#pragma unroll
+        for (int tt = 0; tt < TG; ++tt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                p[tt][r] = sc[tt][r] == -INFINITY ? 0.f : __expf(sc[tt][r] - m_new);
+                sum += p[tt][r];
+            }
+        l_run = l_run * corr + sum;
+        m_run = m_new;
+        return corr;
+    };
 
+    float col_l[MAXU][MAPS];  // a column's whole sum, once it is known
     if constexpr (!TALK) {
-        for (int i = 0; i < n_tiles; ++i) {
-            const int j0 = tile_start(i);
+        for (int round = 0; round < n_rounds; ++round) {
+            const int group = round * NS + slice;
 #pragma unroll
             for (int uu = 0; uu < MAXU; ++uu) {
-                if (wave + uu * nwaves >= a.units) continue;
+                if (!mine[uu]) continue;
+                s16x4 vf[TG][MAXTV];
 #pragma unroll
                 for (int m = 0; m < MAPS; ++m) {
-                    float sc[4];
-                    scores(uu, m, j0, sc);
-                    const float m_new = fmaxf(run_m[uu][m], column_max(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]))));
-                    const float corr = m_new == -INFINITY ? 1.f : __expf(run_m[uu][m] - m_new);
-                    float p[4], sum = 0.f;
+                    float sc[TG][4], p[TG][4];
+                    scores(uu, m, group, sc);
+                    if (m == 0) load_values(uu, group, vf);  // (asked for before the softmax arithmetic; both maps use them)
+                    const float corr = join(sc, run_m[uu][m], run_l[uu][m], p);
+                    s16x4 pf[TG];
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        p[r] = sc[r] == -INFINITY ? 0.f : __expf(sc[r] - m_new);
-                        sum += p[r];
-                    }
-                    run_l[uu][m] = run_l[uu][m] * corr + sum;
-                    run_m[uu][m] = m_new;
+                    for (int tt = 0; tt < TG; ++tt) pf[tt] = pack4(p[tt][0], p[tt][1], p[tt][2], p[tt][3]);
 #pragma unroll
-                    for (int t = 0; t < MAXT; ++t) acc_o[uu][m][t] *= corr;
-                    values(uu, j0, pack4(p[0], p[1], p[2], p[3]), acc_o[uu][m]);
+                    for (int t = 0; t < MAXTV; ++t) acc_o[uu][m][t] *= corr;
+                    times_values(vf, pf, acc_o[uu][m]);
                 }
             }
         }
+#pragma unroll
+        for (int uu = 0; uu < MAXU; ++uu)
+#pragma unroll
+            for (int m = 0; m < MAPS; ++m) col_l[uu][m] = column_sum(run_l[uu][m]);
+        if (NS > 1) {  // the slices of a unit meet in LDS: [unit wave][slice][map]{m[16], l[16], o[dv][16]}
+            const int per = 16 * (2 + dv);
+#pragma unroll
+            for (int uu = 0; uu < MAXU; ++uu)
+#pragma unroll
+                for (int m = 0; m < MAPS; ++m) {
+                    float* mine_at = lds + (size_t)(((uw + uu * n_uw) * NS + slice) * MAPS + m) * per;
+                    if (!mine[uu]) continue;
+                    if (q4 == 0) mine_at[col] = run_m[uu][m], mine_at[16 + col] = col_l[uu][m];
+#pragma unroll
+                    for (int t = 0; t < MAXTV; ++t)
+                        if (t < dvt)
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) mine_at[32 + (16 * t + 4 * q4 + r) * 16 + col] = acc_o[uu][m][t][r];
+                }
+            __syncthreads();
+            if (slice != 0) return;
+#pragma unroll
+            for (int uu = 0; uu < MAXU; ++uu)
+#pragma unroll
+                for (int m = 0; m < MAPS; ++m) {
+                    if (!mine[uu]) continue;
+                    const float* base = lds + (size_t)(((uw + uu * n_uw) * NS) * MAPS + m) * per;
+                    float top = -INFINITY;
+                    for (int s2 = 0; s2 < NS; ++s2) top = fmaxf(top, base[(size_t)s2 * MAPS * per + col]);
+                    float total = 0.f;
+#pragma unroll
+                    for (int t = 0; t < MAXTV; ++t) acc_o[uu][m][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+                    for (int s2 = 0; s2 < NS; ++s2) {
+                        const float* at = base + (size_t)s2 * MAPS * per;
+                        const float f = at[col] == -INFINITY ? 0.f : __expf(at[col] - top);
+                        total += f * at[16 + col];
+#pragma unroll
+                        for (int t = 0; t < MAXTV; ++t)
+                            if (t < dvt)
+#pragma unroll
+                                for (int r = 0; r < 4; ++r) acc_o[uu][m][t][r] += f * at[32 + (16 * t + 4 * q4 + r) * 16 + col];
+                    }
+                    col_l[uu][m] = total;
+                }
+        }
     } else {
-        float* pbuf = lds;                       // [tok][H][16]
-        float* talk_s = lds + a.tok * H * 16;     // [g][h]
+        const int group_keys = 16 * TG;
+        float* pbuf = lds + (size_t)slice * a.tok * H * group_keys;  // [slice][tok][H][16 TG]
+        float* talk_s = lds + (size_t)NS * a.tok * H * group_keys;    // [g][h]
+        float* stats = talk_s + H * H;                               // [unit][slice][2][16]
         for (int i = threadIdx.x; i < H * H; i += blockDim.x) talk_s[(i % H) * H + i / H] = a.talk[i];
         // first walk: every column's maximum and sum
-        for (int i = 0; i < n_tiles; ++i) {
-            const int j0 = tile_start(i);
+        for (int round = 0; round < n_rounds; ++round) {
+            const int group = round * NS + slice;
 #pragma unroll
             for (int uu = 0; uu < MAXU; ++uu) {
-                if (wave + uu * nwaves >= a.units) continue;
-                float sc[4];
-                scores(uu, 0, j0, sc);
-                const float m_new = fmaxf(run_m[uu][0], column_max(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]))));
-                const float corr = m_new == -INFINITY ? 1.f : __expf(run_m[uu][0] - m_new);
-                float sum = 0.f;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) sum += sc[r] == -INFINITY ? 0.f : __expf(sc[r] - m_new);
-                run_l[uu][0] = run_l[uu][0] * corr + sum;
-                run_m[uu][0] = m_new;
+                if (!mine[uu]) continue;
+                float sc[TG][4], p[TG][4];
+                scores(uu, 0, group, sc);
+                join(sc, run_m[uu][0], run_l[uu][0], p);
             }
         }
         float inv_l[MAXU];
 #pragma unroll
-        for (int uu = 0; uu < MAXU; ++uu) inv_l[uu] = 1.f / column_sum(run_l[uu][0]);
+        for (int uu = 0; uu < MAXU; ++uu) col_l[uu][0] = column_sum(run_l[uu][0]);
+        if (NS > 1) {
+#pragma unroll
+            for (int uu = 0; uu < MAXU; ++uu)
+                if (mine[uu] && q4 == 0) {
+                    float* at = stats + (size_t)((uw + uu * n_uw) * NS + slice) * 32;
+                    at[col] = run_m[uu][0], at[16 + col] = col_l[uu][0];
+                }
+            __syncthreads();
+#pragma unroll
+            for (int uu = 0; uu < MAXU; ++uu) {
+                if (!mine[uu]) continue;
+                const float* at = stats + (size_t)((uw + uu * n_uw) * NS) * 32;
+                float top = -INFINITY, total = 0.f;
+                for (int s2 = 0; s2 < NS; ++s2) top = fmaxf(top, at[s2 * 32 + col]);
+                for (int s2 = 0; s2 < NS; ++s2)
+                    total += at[s2 * 32 + col] == -INFINITY ? 0.f : __expf(at[s2 * 32 + col] - top) * at[s2 * 32 + 16 + col];
+                run_m[uu][0] = top, col_l[uu][0] = total;
+            }
+        }
+#pragma unroll
+        for (int uu = 0; uu < MAXU; ++uu) inv_l[uu] = 1.f / col_l[uu][0];
         __syncthreads();  // (the mixing matrix is in LDS)
         // second walk: normalised weights through LDS, mixed, times the values
-        for (int i = 0; i < n_tiles; ++i) {
-            const int j0 = tile_start(i);
+        for (int round = 0; round < n_rounds; ++round) {
+            const int group = round * NS + slice;
+            s16x4 vf[MAXU][TG][MAXTV];
 #pragma unroll
             for (int uu = 0; uu < MAXU; ++uu) {
-                if (wave + uu * nwaves >= a.units) continue;
-                float sc[4];
-                scores(uu, 0, j0, sc);  // (every lane takes part: a padding column's lane still brings a key's row)
-                f32x4 w;
+                if (!mine[uu]) continue;
+                float sc[TG][4];
+                scores(uu, 0, group, sc);
+                load_values(uu, group, vf[uu]);
 #pragma unroll
-                for (int r = 0; r < 4; ++r) w[r] = sc[r] == -INFINITY ? 0.f : __expf(sc[r] - run_m[uu][0]) * inv_l[uu];
-                if (col < a.tpw * a.grp) *reinterpret_cast<f32x4*>(pbuf + ((size_t)u_tl[uu] * H + u_h[uu]) * 16 + 4 * q4) = w;
+                for (int tt = 0; tt < TG; ++tt) {
+                    f32x4 w;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) w[r] = sc[tt][r] == -INFINITY ? 0.f : __expf(sc[tt][r] - run_m[uu][0]) * inv_l[uu];
+                    if (col < used_cols)
+                        *reinterpret_cast<f32x4*>(pbuf + ((size_t)u_tl[uu] * H + u_h[uu]) * group_keys + 16 * tt + 4 * q4) = w;
+                }
             }
             __syncthreads();
 #pragma unroll
             for (int uu = 0; uu < MAXU; ++uu) {
-                if (wave + uu * nwaves >= a.units) continue;
-                f32x4 w = {0.f, 0.f, 0.f, 0.f};
-                if (col < a.tpw * a.grp) {
-                    const float* prow = pbuf + (size_t)u_tl[uu] * H * 16 + 4 * q4;
+                if (!mine[uu]) continue;
+                f32x4 w[TG];
+#pragma unroll
+                for (int tt = 0; tt < TG; ++tt) w[tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+                if (col < used_cols) {
+                    const float* prow = pbuf + (size_t)u_tl[uu] * H * group_keys + 4 * q4;
                     const float* trow = talk_s + u_h[uu];
                     for (int g = 0; g < H; ++g) {
-                        const f32x4 pg = *reinterpret_cast<const f32x4*>(prow + g * 16);
                         const float tg = trow[g * H];
-                        w += tg * pg;
+#pragma unroll
+                        for (int tt = 0; tt < TG; ++tt) w[tt] += tg * *reinterpret_cast<const f32x4*>(prow + g * group_keys + 16 * tt);
                     }
                 }
-                values(uu, j0, pack4(w[0], w[1], w[2], w[3]), acc_o[uu][0]);
+                s16x4 pf[TG];
+#pragma unroll
+                for (int tt = 0; tt < TG; ++tt) pf[tt] = pack4(w[tt][0], w[tt][1], w[tt][2], w[tt][3]);
+                times_values(vf[uu], pf, acc_o[uu][0]);
             }
             __syncthreads();
+        }
+        if (NS > 1) {  // the slices' partial results, already normalised, add up: [unit][slice][dv][16] over the weights' place
+            float* sums = lds;
+            const int per = 16 * dv;
+#pragma unroll
+            for (int uu = 0; uu < MAXU; ++uu) {
+                if (!mine[uu]) continue;
+                float* at = sums + (size_t)((uw + uu * n_uw) * NS + slice) * per;
+#pragma unroll
+                for (int t = 0; t < MAXTV; ++t)
+                    if (t < dvt)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) at[(16 * t + 4 * q4 + r) * 16 + col] = acc_o[uu][0][t][r];
+            }
+            __syncthreads();
+            if (slice != 0) return;
+#pragma unroll
+            for (int uu = 0; uu < MAXU; ++uu) {
+                if (!mine[uu]) continue;
+                const float* at = sums + (size_t)((uw + uu * n_uw) * NS) * per;
+                for (int s2 = 1; s2 < NS; ++s2)
+#pragma unroll
+                    for (int t = 0; t < MAXTV; ++t)
+                        if (t < dvt)
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) acc_o[uu][0][t][r] += at[(size_t)s2 * per + (16 * t + 4 * q4 + r) * 16 + col];
+            }
         }
     }
 
     // what leaves: per column, 4 neighbouring dimensions per tile of 16
 #pragma unroll
     for (int uu = 0; uu < MAXU; ++uu) {
-        if (wave + uu * nwaves >= a.units) continue;
+        if (!mine[uu]) continue;
         float mul[MAPS];
 #pragma unroll
-        for (int m = 0; m < MAPS; ++m) mul[m] = TALK ? 1.f : 1.f / column_sum(run_l[uu][m]);
+        for (int m = 0; m < MAPS; ++m) mul[m] = TALK ? 1.f : 1.f / col_l[uu][m];
         float ss = 0.f;
 #pragma unroll
-        for (int t = 0; t < MAXT; ++t)
+        for (int t = 0; t < MAXTV; ++t)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 float o = acc_o[uu][0][t][r] * mul[0];
@@ -272,7 +419,7 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
         if (!valid[uu]) continue;
         bf16* orow = a.out + (size_t)(row0 + t0 + u_tl[uu]) * a.out_stride + (size_t)u_h[uu] * dv + 4 * q4;
 #pragma unroll
-        for (int t = 0; t < MAXT; ++t)
+        for (int t = 0; t < MAXTV; ++t)
             if (t < dvt) {
                 const f32x4 o = acc_o[uu][0][t] * norm;
                 *reinterpret_cast<s16x4*>(orow + 16 * t) = pack4(o[0], o[1], o[2], o[3]);
@@ -280,20 +427,24 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
     }
 }
 
+// tiles in a group: 4 (64 keys) up to sizes of 64; wider keys or values leave registers for 2
+#define AM_TG 4
+#define AM_TG_WIDE 2
+
 template <int MAPS, bool TALK, int MAXU, int THREADS>
 static int launch(const MfmaArgs& a, dim3 grid, int threads, size_t lds, hipStream_t stream) {
-    const int tiles = (a.dk > a.dv ? a.dk : a.dv) / 16;
-    if (tiles <= 4) {
-        auto kernel = attend_mfma_kernel<MAPS, TALK, 4, MAXU, THREADS>;
-        if (lds > 48 * 1024)
-            LLMS_HIP_CHECK(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        kernel<<<grid, threads, lds, stream>>>(a);
-    } else {
-        auto kernel = attend_mfma_kernel<MAPS, TALK, 8, MAXU, THREADS>;
-        if (lds > 48 * 1024)
-            LLMS_HIP_CHECK(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        kernel<<<grid, threads, lds, stream>>>(a);
-    }
+#define AM_LAUNCH(TK, TV)                                                                                              \
+    do {                                                                                                               \
+        auto kernel = attend_mfma_kernel<MAPS, TALK, TK, TV, MAXU, (TK > 4 || TV > 4) ? AM_TG_WIDE : AM_TG, THREADS>;  \
+        if (lds > 48 * 1024)                                                                                           \
+            LLMS_HIP_CHECK(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
+        kernel<<<grid, threads, lds, stream>>>(a);                                                                     \
+    } while (0)
+    if (a.dk <= 64 && a.dv <= 64) AM_LAUNCH(4, 4);
+    else if (a.dk <= 64) AM_LAUNCH(4, 8);
+    else if (a.dv <= 64) AM_LAUNCH(8, 4);
+    else AM_LAUNCH(8, 8);
+#undef AM_LAUNCH
     LLMS_LAUNCH_CHECK();
 }
 
@@ -324,15 +475,25 @@ int llms_attend_composed_mfma(void* out, int out_stride, const void* q, int q_st
     a.window = window, a.keep_first = keep_first, a.chunk = chunk;
     a.scale = scale, a.lambda = lambda, a.eps = eps, a.out_scale = out_scale, a.head_norm = head_norm;
     a.tpw = 16 / a.grp;
+    const int group_keys = 16 * ((dk > 64 || dv > 64) ? AM_TG_WIDE : AM_TG);
     if (talk) {
         LLMS_REQUIRE(kv_heads <= 32, "attend_composed_mfma: mixing heads takes up to 32 key/value heads");
-        // every head of a block of tokens in one workgroup: up to 32 units in up to 16 waves
+        // every head of a block of tokens in one workgroup: up to 32 units in up to 16 waves, the normalised
+        // weights of a group of keys in up to 64 KB of LDS (more only if a single unit per key/value head needs it)
         int upk = 32 / kv_heads;
+        while (upk > 1 && (size_t)upk * a.tpw * heads * group_keys * sizeof(float) > 64 * 1024) --upk;
         while (upk > 1 && (upk - 1) * a.tpw >= max_new) --upk;  // (no more tokens than the longest portion has)
         a.upk = upk, a.tok = upk * a.tpw, a.kv_per_wg = kv_heads, a.units = kv_heads * upk;
-        const int waves = a.units > 16 ? (a.units + 1) / 2 : a.units;
+        a.slices = 1;
+        if (upk == 1)  // few tokens (decoding): the groups of keys are dealt to several waves per unit
+            while (a.slices < 4 && a.units * a.slices * 2 <= 16) a.slices *= 2;
+        const int unit_waves = a.units > 16 ? (a.units + 1) / 2 : a.units;
+        const int waves = unit_waves * a.slices;
         a.blocks_per_seq = (max_new + a.tok - 1) / a.tok;
-        const size_t lds = ((size_t)a.tok * heads * 16 + (size_t)heads * heads) * sizeof(float);
+        size_t floats = (size_t)a.slices * a.tok * heads * group_keys + (size_t)heads * heads + (size_t)a.units * a.slices * 32;
+        const size_t merge = a.slices > 1 ? (size_t)a.units * a.slices * 16 * dv : 0;
+        if (merge > floats) floats = merge;
+        const size_t lds = floats * sizeof(float);
         LLMS_REQUIRE(lds <= 160 * 1024, "attend_composed_mfma: too many heads for the LDS");
         dim3 grid(n_seqs * a.blocks_per_seq, 1);
         if (a.units > 16) return launch<1, true, 2, 1024>(a, grid, waves * LLMS_WAVE, lds, stream);
@@ -341,11 +502,13 @@ int llms_attend_composed_mfma(void* out, int out_stride, const void* q, int q_st
     int upk = 4;
     while (upk > 1 && (upk - 1) * a.tpw >= max_new) --upk;
     a.upk = upk, a.tok = upk * a.tpw, a.kv_per_wg = 1, a.units = upk;
+    a.slices = upk == 1 ? 4 : 1;
     a.blocks_per_seq = (max_new + a.tok - 1) / a.tok;
+    const size_t lds = a.slices > 1 ? (size_t)a.units * a.slices * maps * 16 * (2 + dv) * sizeof(float) : 0;
     dim3 grid(n_seqs * a.blocks_per_seq, kv_heads);
     LLMS_REQUIRE(grid.y <= 65535, "attend_composed_mfma: too many key/value heads");
-    if (maps == 2) return launch<2, false, 1, 256>(a, grid, upk * LLMS_WAVE, 0, stream);
-    return launch<1, false, 1, 256>(a, grid, upk * LLMS_WAVE, 0, stream);
+    if (maps == 2) return launch<2, false, 1, 256>(a, grid, upk * a.slices * LLMS_WAVE, lds, stream);
+    return launch<1, false, 1, 256>(a, grid, upk * a.slices * LLMS_WAVE, lds, stream);
 }
 
 }  // extern "C"
