@@ -195,13 +195,15 @@ DESIGN_SIZES = {  # layer sizes of the named Llama shapes
 
 
 def dibepel_config(size: dict, layers: int, window: int = 1024, keep_first: int = 64, chunk: int = 1024, taps: int = 4) -> dict:
-    """Every third layer the windowed attention with two score maps (half the heads, values twice as wide, so that
-    its projections have the sizes of the others'), the rest the chunked attention with convolutions and mixed heads."""
+    """Every third layer the windowed attention with two score maps (half the heads, values twice as wide up to 128, so
+    that its projections have the sizes of the others'), the rest the chunked attention with convolutions and mixed
+    heads."""
     entries = []
     for i in range(layers):
         if i % 3 == 2:
+            # (values twice as wide where that stays within the 128 the matrix-core attention takes)
             mixer = {"heads": size["heads"] // 2, "kv_heads": max(1, size["kv_heads"] // 2), "dim": size["dim"],
-                     "vdim": 2 * size["dim"], "diff": 0.5, "scale": size["dim"] ** -0.5,
+                     "vdim": min(2 * size["dim"], 128), "diff": 0.5, "scale": size["dim"] ** -0.5,
                      "mask": {"size": window, "keep_first": keep_first}}
             kind = "attention"
         else:

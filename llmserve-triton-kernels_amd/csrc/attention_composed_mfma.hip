@@ -29,6 +29,11 @@
 // were given back (table entry < 0) and values behind the request's end are read as zeros.
 #include "common.h"
 
+#define AM_PAGE_CACHE 1024  // page ids (4 bytes each) a workgroup keeps in LDS
+
+#define LOG2E 1.4426950408889634f
+#define NOTHING_YET (-1.0e30f)
+
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
@@ -48,9 +53,18 @@ struct MfmaArgs {
     int heads, kv_heads, grp, dk, dv, block_size;
     int window, keep_first, chunk;
     int tok, tpw, upk, units, kv_per_wg, slices;
+    unsigned bs_magic;  // ceil(2^32 / block_size): key / block_size is one multiply-high
+    // a request's keys shared out to `shares` workgroups (grid z), with TALK: mode 1 leaves every column's maximum and
+    // sum over its share in ws_stats [row][head][share][2] and ends; mode 2 takes them from there, walks its share once
+    // more and leaves its part of the result, 32-bit, in ws_o [share][row][heads * dv]; a last kernel adds the parts up
+    int shares, mode, ws_rows;
+    float* ws_stats;
+    float* ws_o;
     float scale, lambda, eps, out_scale;
     int head_norm;
 };
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }  // v_exp_f32; 0 for -inf
 
 __device__ __forceinline__ s16x4 load4(const bf16* p) { return *reinterpret_cast<const s16x4*>(p); }
 
@@ -72,7 +86,9 @@ __device__ __forceinline__ float column_sum(float v) {
 
 template <int MAPS, bool TALK, int MAXTK, int MAXTV, int MAXU, int TG, int THREADS>
 __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) {
-    extern __shared__ float lds[];
+    extern __shared__ float lds_all[];
+    int* pages_s = reinterpret_cast<int*>(lds_all);  // the request's page ids over the keys this workgroup walks
+    float* lds = lds_all + AM_PAGE_CACHE;
     const int wave = threadIdx.x / LLMS_WAVE, lane = threadIdx.x % LLMS_WAVE, nwaves = blockDim.x / LLMS_WAVE;
     const int col = lane % 16, q4 = lane / 16;
     const int NS = a.slices, slice = wave % NS, uw = wave / NS, n_uw = nwaves / NS;
@@ -100,7 +116,23 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
     const int n_sink = sink_end - sink_begin;
     const int n_tiles = n_sink + (main_end - main_begin);
     const int n_groups = (n_tiles + TG - 1) / TG;
-    const int n_rounds = (n_groups + NS - 1) / NS;  // every slice walks this many groups (the last may be empty)
+    const int NSG = a.shares, share = blockIdx.z;
+    const int n_rounds = (n_groups + NS * NSG - 1) / (NS * NSG);  // every slice walks this many groups (the last may be empty)
+    // groups behind this one hold only tiles whose keys the first token reaches: their pages are all there
+    const int first_plain = n_sink / TG + 1;
+    // the pages of the walked keys (those from the first reachable key on; up to AM_PAGE_CACHE of them) are read once
+    const int first_block = (int)__umulhi((unsigned)(main_begin * 16), a.bs_magic);
+    int cached = (int)__umulhi((unsigned)end, a.bs_magic) + 1 - first_block;
+    if (cached > AM_PAGE_CACHE) cached = AM_PAGE_CACHE;
+    for (int i = threadIdx.x; i < cached; i += blockDim.x) pages_s[i] = first_block + i < a.max_blocks ? table[first_block + i] : -1;
+    __syncthreads();
+    // (one load through a pointer chosen between LDS and memory: no branch stands between the loads of a group)
+    auto block_of = [&](int key) { return (int)__umulhi((unsigned)key, a.bs_magic); };
+    auto page_at = [&](int block) {
+        const int i = block - first_block;
+        const int* at = (i >= 0 && i < cached) ? static_cast<const int*>(pages_s + i) : table + block;
+        return *at;
+    };
     // first key of tile i; tiles behind the last lie behind every token's position and hold nothing
     auto tile_start = [&](int i) { return 16 * (i < n_sink ? sink_begin + i : main_begin + (i - n_sink)); };
 
@@ -108,6 +140,7 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
     bool valid[MAXU], mine[MAXU];
     int u_kvh[MAXU], u_h[MAXU], u_tl[MAXU], u_pos[MAXU], u_chunk_lo[MAXU];
     float u_slope[MAXU];
+    int u_pmin[MAXU], u_pmax[MAXU];
     s16x4 qf[MAXU][MAPS][MAXTK];
 #pragma unroll
     for (int uu = 0; uu < MAXU; ++uu) {
@@ -118,61 +151,99 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
         valid[uu] = mine[uu] && col < used_cols && tl < ntok;
         u_kvh[uu] = kvh, u_h[uu] = h, u_tl[uu] = tl, u_pos[uu] = pos_lo + tl;
         u_chunk_lo[uu] = a.chunk > 0 ? u_pos[uu] / a.chunk * a.chunk : 0;
-        u_slope[uu] = (a.slopes && valid[uu]) ? a.slopes[h] : 0.f;
+        u_slope[uu] = (a.slopes && valid[uu]) ? a.slopes[h] * LOG2E : 0.f;
+        // the unit's first and last position (the same for all its lanes): a tile that all of them see whole
+        // needs no comparisons
+        u_pmin[uu] = pos_lo + sub * a.tpw;
+        u_pmax[uu] = u_pmin[uu] + a.tpw - 1 < pos_hi ? u_pmin[uu] + a.tpw - 1 : pos_hi;
         const bf16* qrow = a.q + (size_t)(row0 + t0 + tl) * a.q_stride + (size_t)h * MAPS * dk + 4 * q4;
 #pragma unroll
         for (int m = 0; m < MAPS; ++m)
 #pragma unroll
             for (int t = 0; t < MAXTK; ++t)
-                qf[uu][m][t] = (valid[uu] && t < dkt) ? load4(qrow + m * dk + 16 * t) : s16x4{0, 0, 0, 0};
+                qf[uu][m][t] = (valid[uu] && t < dkt) ? load4(qrow + m * dk + 16 * t) : s16x4{0, 0, 0, 0};  // (once; rows of padding are not read)
     }
 
     // scores of one group of tiles for one unit and map: per tile 4 keys (j0 + 4 q4 + r) of the lane's column,
     // masked to -inf.  Every lane takes part, also one whose column is padding: it still brings a key's row.
+    // scores are kept in units of log 2 (scale and slopes carry the factor), so a weight is one subtraction and one
+    // v_exp_f32; a maximum of -inf (nothing seen yet) is replaced by a large negative number, so that exp2(-inf - m) is 0
+    const float scale2 = a.scale * LOG2E;
+    const size_t k_page = (size_t)G * MAPS * bs * dk, v_page = (size_t)G * dv * bs;  // elements in a page
     auto scores = [&](int uu, int m, int group, float sc[TG][4]) {
         s16x4 kf[TG][MAXTK];
+        const bf16* kbase = a.k_pool + (size_t)(u_kvh[uu] * MAPS + m) * bs * dk + 4 * q4;
 #pragma unroll
         for (int tt = 0; tt < TG; ++tt) {
             const int j = tile_start(group * TG + tt) + col;  // the key whose row this lane brings
-            const int page = j <= pos_hi ? table[j / bs] : -1;
-            const bf16* krow = a.k_pool + (((size_t)(page < 0 ? 0 : page) * (G * MAPS) + u_kvh[uu] * MAPS + m) * bs + j % bs) * dk + 4 * q4;
+            // every load is issued whatever it brings (a key that is not there reads the request's first row and is
+            // replaced by zeros afterwards): a branch around a load would make the wave wait for all loads in flight
+            const int jj = j <= pos_hi ? j : pos_lo;
+            const int block = block_of(jj);
+            const int got = page_at(block);
+            const int page = j <= pos_hi ? got : -1;
+            const bf16* krow = kbase + (size_t)(page < 0 ? 0 : page) * k_page + (jj - block * bs) * dk;
+            // (a group that lies among the reachable keys, with keys as wide as the kernel's tiles, needs no zeros)
+            const bool plain_k = dkt == MAXTK && group > first_plain && tile_start(group * TG + TG - 1) + 15 <= pos_hi;
 #pragma unroll
-            for (int t = 0; t < MAXTK; ++t) kf[tt][t] = (page >= 0 && t < dkt) ? load4(krow + 16 * t) : s16x4{0, 0, 0, 0};
+            for (int t = 0; t < MAXTK; ++t) {
+                const s16x4 k = load4(krow + (t < dkt ? 16 * t : 0));
+                kf[tt][t] = (plain_k || (page >= 0 && t < dkt)) ? k : s16x4{0, 0, 0, 0};
+            }
         }
         const int pos = u_pos[uu];
 #pragma unroll
         for (int tt = 0; tt < TG; ++tt) {
             f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int t = 0; t < MAXTK; ++t)
-                if (t < dkt) acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kf[tt][t], qf[uu][m][t], acc, 0, 0, 0);
+            for (int t = 0; t < MAXTK; ++t)  // (tiles beyond the keys' size hold zeros)
+                acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kf[tt][t], qf[uu][m][t], acc, 0, 0, 0);
             const int j0 = tile_start(group * TG + tt);
+            const float dist0 = (float)(pos - j0 - 4 * q4);
+            // all the unit's positions see all 16 keys (the same answer in every lane): no comparison per key; a
+            // column of padding then holds numbers that nobody reads
+            const bool whole = j0 + 15 <= u_pmin[uu] && (a.chunk <= 0 || j0 >= u_pmax[uu] / a.chunk * a.chunk) &&
+                               (a.window <= 0 || u_pmax[uu] - j0 < a.window);
+            if (whole) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int key = j0 + 4 * q4 + r;
-                const bool vis = valid[uu] && key <= pos && key >= u_chunk_lo[uu] &&
-                                 (a.window <= 0 || pos - key < a.window || key < a.keep_first);
-                sc[tt][r] = vis ? acc[r] * a.scale - u_slope[uu] * (float)(pos - key) : -INFINITY;
+                for (int r = 0; r < 4; ++r) sc[tt][r] = acc[r] * scale2 - u_slope[uu] * (dist0 - (float)r);
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int key = j0 + 4 * q4 + r;
+                    const bool vis = valid[uu] && key <= pos && key >= u_chunk_lo[uu] &&
+                                     (a.window <= 0 || pos - key < a.window || key < a.keep_first);
+                    sc[tt][r] = vis ? acc[r] * scale2 - u_slope[uu] * (dist0 - (float)r) : -INFINITY;
+                }
             }
         }
     };
     // the values of key/value head u_kvh for one group: per tile, keys j0 + 4 q4 .. + 3 of dimension 16 t + col
     auto load_values = [&](int uu, int group, s16x4 vf[TG][MAXTV]) {
+        const bf16* vbase = a.v_pool + ((size_t)u_kvh[uu] * dv + col) * bs;
 #pragma unroll
         for (int tt = 0; tt < TG; ++tt) {
             const int key = tile_start(group * TG + tt) + 4 * q4;
-            const int page = key < end ? table[key / bs] : -1;
+            const int kk = key < end ? key : pos_lo / 4 * 4;
+            const int block = block_of(kk);
+            const int got = page_at(block);
+            const int page = key < end ? got : -1;
             const int keep = end - key;  // keys behind the request's end hold nothing
-            const bf16* vrow = a.v_pool + (((size_t)(page < 0 ? 0 : page) * G + u_kvh[uu]) * dv + col) * bs + key % bs;
+            const bf16* vrow = vbase + (size_t)(page < 0 ? 0 : page) * v_page + (kk - block * bs);
+            const bool plain_v = dvt == MAXTV && group > first_plain && tile_start(group * TG + TG - 1) + 15 < end;
+            if (plain_v) {
 #pragma unroll
-            for (int t = 0; t < MAXTV; ++t) {
-                s16x4 v = (page >= 0 && t < dvt) ? load4(vrow + (size_t)16 * t * bs) : s16x4{0, 0, 0, 0};
-                if (keep < 4) {
-                    if (keep < 2) v.y = 0;
-                    if (keep < 3) v.z = 0;
-                    v.w = 0;
+                for (int t = 0; t < MAXTV; ++t) vf[tt][t] = load4(vrow + (size_t)16 * t * bs);
+            } else {
+#pragma unroll
+                for (int t = 0; t < MAXTV; ++t) {
+                    const s16x4 got_v = load4(vrow + (t < dvt ? (size_t)16 * t * bs : 0));
+                    s16x4 v = (page >= 0 && t < dvt) ? got_v : s16x4{0, 0, 0, 0};
+                    v.y = keep < 2 ? (short)0 : v.y;
+                    v.z = keep < 3 ? (short)0 : v.z;
+                    v.w = keep < 4 ? (short)0 : v.w;
+                    vf[tt][t] = v;
                 }
-                vf[tt][t] = v;
             }
         }
     };
@@ -180,8 +251,7 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
 #pragma unroll
         for (int tt = 0; tt < TG; ++tt)
 #pragma unroll
-            for (int t = 0; t < MAXTV; ++t)
-                if (t < dvt) o[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf[tt][t], pf[tt], o[t], 0, 0, 0);
+            for (int t = 0; t < MAXTV; ++t) o[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf[tt][t], pf[tt], o[t], 0, 0, 0);
     };
 
     f32x4 acc_o[MAXU][MAPS][MAXTV];
@@ -190,7 +260,7 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
     for (int uu = 0; uu < MAXU; ++uu)
 #pragma unroll
         for (int m = 0; m < MAPS; ++m) {
-            run_m[uu][m] = -INFINITY, run_l[uu][m] = 0.f;
+            run_m[uu][m] = NOTHING_YET, run_l[uu][m] = 0.f;
 #pragma unroll
             for (int t = 0; t < MAXTV; ++t) acc_o[uu][m][t] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
@@ -201,14 +271,14 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
         for (int tt = 0; tt < TG; ++tt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) mx = fmaxf(mx, sc[tt][r]);
-        const float m_new = fmaxf(m_run, column_max(mx));
-        const float corr = m_new == -INFINITY ? 1.f : __expf(m_run - m_new);
+        const float m_new = fmaxf(fmaxf(m_run, column_max(mx)), NOTHING_YET);
+        const float corr = fast_exp2(m_run - m_new);
         float sum = 0.f;
 #pragma unroll
         for (int tt = 0; tt < TG; ++tt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                p[tt][r] = sc[tt][r] == -INFINITY ? 0.f : __expf(sc[tt][r] - m_new);
+                p[tt][r] = fast_exp2(sc[tt][r] - m_new);
                 sum += p[tt][r];
             }
         l_run = l_run * corr + sum;
@@ -219,7 +289,8 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
     float col_l[MAXU][MAPS];  // a column's whole sum, once it is known
     if constexpr (!TALK) {
         for (int round = 0; round < n_rounds; ++round) {
-            const int group = round * NS + slice;
+            const int group = (round * NS + slice) * NSG + share;
+            if (group >= n_groups) break;  // (nothing left for this slice)
 #pragma unroll
             for (int uu = 0; uu < MAXU; ++uu) {
                 if (!mine[uu]) continue;
@@ -227,8 +298,8 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
 #pragma unroll
                 for (int m = 0; m < MAPS; ++m) {
                     float sc[TG][4], p[TG][4];
+                    if (m == 0) load_values(uu, group, vf);  // (asked for beside the keys; both maps use them)
                     scores(uu, m, group, sc);
-                    if (m == 0) load_values(uu, group, vf);  // (asked for before the softmax arithmetic; both maps use them)
                     const float corr = join(sc, run_m[uu][m], run_l[uu][m], p);
                     s16x4 pf[TG];
 #pragma unroll
@@ -266,14 +337,14 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
                 for (int m = 0; m < MAPS; ++m) {
                     if (!mine[uu]) continue;
                     const float* base = lds + (size_t)(((uw + uu * n_uw) * NS) * MAPS + m) * per;
-                    float top = -INFINITY;
+                    float top = NOTHING_YET;
                     for (int s2 = 0; s2 < NS; ++s2) top = fmaxf(top, base[(size_t)s2 * MAPS * per + col]);
                     float total = 0.f;
 #pragma unroll
                     for (int t = 0; t < MAXTV; ++t) acc_o[uu][m][t] = f32x4{0.f, 0.f, 0.f, 0.f};
                     for (int s2 = 0; s2 < NS; ++s2) {
                         const float* at = base + (size_t)s2 * MAPS * per;
-                        const float f = at[col] == -INFINITY ? 0.f : __expf(at[col] - top);
+                        const float f = fast_exp2(at[col] - top);
                         total += f * at[16 + col];
 #pragma unroll
                         for (int t = 0; t < MAXTV; ++t)
@@ -291,8 +362,9 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
         float* stats = talk_s + H * H;                               // [unit][slice][2][16]
         for (int i = threadIdx.x; i < H * H; i += blockDim.x) talk_s[(i % H) * H + i / H] = a.talk[i];
         // first walk: every column's maximum and sum
-        for (int round = 0; round < n_rounds; ++round) {
-            const int group = round * NS + slice;
+        for (int round = 0; round < (a.mode == 2 ? 0 : n_rounds); ++round) {
+            const int group = (round * NS + slice) * NSG + share;
+            if (group >= n_groups) break;  // (nothing left for this slice)
 #pragma unroll
             for (int uu = 0; uu < MAXU; ++uu) {
                 if (!mine[uu]) continue;
@@ -316,10 +388,30 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
             for (int uu = 0; uu < MAXU; ++uu) {
                 if (!mine[uu]) continue;
                 const float* at = stats + (size_t)((uw + uu * n_uw) * NS) * 32;
-                float top = -INFINITY, total = 0.f;
+                float top = NOTHING_YET, total = 0.f;
                 for (int s2 = 0; s2 < NS; ++s2) top = fmaxf(top, at[s2 * 32 + col]);
-                for (int s2 = 0; s2 < NS; ++s2)
-                    total += at[s2 * 32 + col] == -INFINITY ? 0.f : __expf(at[s2 * 32 + col] - top) * at[s2 * 32 + 16 + col];
+                for (int s2 = 0; s2 < NS; ++s2) total += fast_exp2(at[s2 * 32 + col] - top) * at[s2 * 32 + 16 + col];
+                run_m[uu][0] = top, col_l[uu][0] = total;
+            }
+        }
+        if (a.mode == 1) {  // this share's maxima and sums go to memory; the second walk is another launch
+#pragma unroll
+            for (int uu = 0; uu < MAXU; ++uu)
+                if (valid[uu] && q4 == 0 && slice == 0) {
+                    float* at = a.ws_stats + (((size_t)(row0 + t0 + u_tl[uu]) * H + u_h[uu]) * NSG + share) * 2;
+                    at[0] = run_m[uu][0], at[1] = col_l[uu][0];
+                }
+            return;
+        }
+        if (a.mode == 2) {
+#pragma unroll
+            for (int uu = 0; uu < MAXU; ++uu) {
+                float top = NOTHING_YET, total = 0.f;
+                if (valid[uu]) {
+                    const float* at = a.ws_stats + ((size_t)(row0 + t0 + u_tl[uu]) * H + u_h[uu]) * NSG * 2;
+                    for (int s2 = 0; s2 < NSG; ++s2) top = fmaxf(top, at[2 * s2]);
+                    for (int s2 = 0; s2 < NSG; ++s2) total += fast_exp2(at[2 * s2] - top) * at[2 * s2 + 1];
+                }
                 run_m[uu][0] = top, col_l[uu][0] = total;
             }
         }
@@ -328,19 +420,20 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
         __syncthreads();  // (the mixing matrix is in LDS)
         // second walk: normalised weights through LDS, mixed, times the values
         for (int round = 0; round < n_rounds; ++round) {
-            const int group = round * NS + slice;
+            const int group = (round * NS + slice) * NSG + share;
+            const bool some = group < n_groups;  // (a slice without keys in this round only keeps the barriers' count)
             s16x4 vf[MAXU][TG][MAXTV];
 #pragma unroll
             for (int uu = 0; uu < MAXU; ++uu) {
-                if (!mine[uu]) continue;
+                if (!mine[uu] || !some) continue;
                 float sc[TG][4];
-                scores(uu, 0, group, sc);
                 load_values(uu, group, vf[uu]);
+                scores(uu, 0, group, sc);
 #pragma unroll
                 for (int tt = 0; tt < TG; ++tt) {
                     f32x4 w;
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) w[r] = sc[tt][r] == -INFINITY ? 0.f : __expf(sc[tt][r] - run_m[uu][0]) * inv_l[uu];
+                    for (int r = 0; r < 4; ++r) w[r] = fast_exp2(sc[tt][r] - run_m[uu][0]) * inv_l[uu];
                     if (col < used_cols)
                         *reinterpret_cast<f32x4*>(pbuf + ((size_t)u_tl[uu] * H + u_h[uu]) * group_keys + 16 * tt + 4 * q4) = w;
                 }
@@ -348,7 +441,7 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
             __syncthreads();
 #pragma unroll
             for (int uu = 0; uu < MAXU; ++uu) {
-                if (!mine[uu]) continue;
+                if (!mine[uu] || !some) continue;
                 f32x4 w[TG];
 #pragma unroll
                 for (int tt = 0; tt < TG; ++tt) w[tt] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -417,6 +510,13 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
         float norm = 1.f;
         if (a.head_norm) norm = a.out_scale / sqrtf(column_sum(ss) / (float)dv + a.eps);
         if (!valid[uu]) continue;
+        if (TALK && a.mode == 2) {  // this share's part, unrounded
+            float* part = a.ws_o + ((size_t)share * a.ws_rows + row0 + t0 + u_tl[uu]) * ((size_t)H * dv) + (size_t)u_h[uu] * dv + 4 * q4;
+#pragma unroll
+            for (int t = 0; t < MAXTV; ++t)
+                if (t < dvt) *reinterpret_cast<f32x4*>(part + 16 * t) = acc_o[uu][0][t];
+            continue;
+        }
         bf16* orow = a.out + (size_t)(row0 + t0 + u_tl[uu]) * a.out_stride + (size_t)u_h[uu] * dv + 4 * q4;
 #pragma unroll
         for (int t = 0; t < MAXTV; ++t)
@@ -424,6 +524,20 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
                 const f32x4 o = acc_o[uu][0][t] * norm;
                 *reinterpret_cast<s16x4*>(orow + 16 * t) = pack4(o[0], o[1], o[2], o[3]);
             }
+    }
+}
+
+// out[row] = the sum of the shares' parts, rounded once; one workgroup per request of one token
+__global__ __launch_bounds__(256) void add_shares_kernel(bf16* __restrict__ out, int out_stride, const float* __restrict__ ws_o,
+                                                         int ws_rows, int shares, int width, const int* __restrict__ cu_seqlens,
+                                                         const int* __restrict__ context_lens, int seq_begin) {
+    const int b = seq_begin + blockIdx.x;
+    if (context_lens[b] <= 0) return;
+    const int row = cu_seqlens[b];
+    for (int c = 4 * threadIdx.x; c < width; c += 4 * 256) {
+        f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+        for (int s2 = 0; s2 < shares; ++s2) sum += *reinterpret_cast<const f32x4*>(ws_o + ((size_t)s2 * ws_rows + row) * width + c);
+        *reinterpret_cast<s16x4*>(out + (size_t)row * out_stride + c) = pack4(sum[0], sum[1], sum[2], sum[3]);
     }
 }
 
@@ -456,7 +570,8 @@ int llms_attend_composed_mfma(void* out, int out_stride, const void* q, int q_st
                               const int* cu_seqlens, const int* context_lens, int seq_begin, int n_seqs, int max_new,
                               int heads, int kv_heads, int maps, int dk, int dv, int block_size, int window,
                               int keep_first, int chunk, float scale, const float* slopes, const float* talk, float lambda,
-                              int head_norm, float eps, float out_scale, hipStream_t stream) {
+                              int head_norm, float eps, float out_scale, int shares, float* ws_stats, float* ws_o, int ws_rows,
+                              hipStream_t stream) {
     LLMS_REQUIRE(n_seqs > 0 && max_new > 0 && heads > 0 && kv_heads > 0, "attend_composed_mfma: sizes must be positive");
     LLMS_REQUIRE(heads % kv_heads == 0 && heads / kv_heads <= 16, "attend_composed_mfma: up to 16 query heads per key/value head");
     LLMS_REQUIRE(maps == 1 || maps == 2, "attend_composed_mfma: one or two score maps");
@@ -475,6 +590,8 @@ int llms_attend_composed_mfma(void* out, int out_stride, const void* q, int q_st
     a.window = window, a.keep_first = keep_first, a.chunk = chunk;
     a.scale = scale, a.lambda = lambda, a.eps = eps, a.out_scale = out_scale, a.head_norm = head_norm;
     a.tpw = 16 / a.grp;
+    a.shares = 1, a.mode = 0, a.ws_stats = ws_stats, a.ws_o = ws_o, a.ws_rows = ws_rows;
+    a.bs_magic = (unsigned)((0x100000000ull + block_size - 1) / block_size);
     const int group_keys = 16 * ((dk > 64 || dv > 64) ? AM_TG_WIDE : AM_TG);
     if (talk) {
         LLMS_REQUIRE(kv_heads <= 32, "attend_composed_mfma: mixing heads takes up to 32 key/value heads");
@@ -493,9 +610,22 @@ int llms_attend_composed_mfma(void* out, int out_stride, const void* q, int q_st
         size_t floats = (size_t)a.slices * a.tok * heads * group_keys + (size_t)heads * heads + (size_t)a.units * a.slices * 32;
         const size_t merge = a.slices > 1 ? (size_t)a.units * a.slices * 16 * dv : 0;
         if (merge > floats) floats = merge;
-        const size_t lds = floats * sizeof(float);
+        const size_t lds = (floats + AM_PAGE_CACHE) * sizeof(float);
         LLMS_REQUIRE(lds <= 160 * 1024, "attend_composed_mfma: too many heads for the LDS");
         dim3 grid(n_seqs * a.blocks_per_seq, 1);
+        if (shares > 1 && upk == 1 && max_new == 1) {  // single tokens: every request's keys go to `shares` workgroups
+            LLMS_REQUIRE(ws_stats && ws_o && ws_rows > 0 && shares <= 64, "attend_composed_mfma: shares need their workspaces");
+            a.shares = shares;
+            grid.z = shares;
+            for (a.mode = 1; a.mode <= 2; ++a.mode) {
+                const int rc = a.units > 16 ? launch<1, true, 2, 1024>(a, grid, waves * LLMS_WAVE, lds, stream)
+                                            : launch<1, true, 1, 1024>(a, grid, waves * LLMS_WAVE, lds, stream);
+                if (rc != LLMS_OK) return rc;
+            }
+            add_shares_kernel<<<n_seqs, 256, 0, stream>>>(a.out, out_stride, ws_o, ws_rows, shares, heads * dv, cu_seqlens,
+                                                          context_lens, seq_begin);
+            LLMS_LAUNCH_CHECK();
+        }
         if (a.units > 16) return launch<1, true, 2, 1024>(a, grid, waves * LLMS_WAVE, lds, stream);
         return launch<1, true, 1, 1024>(a, grid, waves * LLMS_WAVE, lds, stream);
     }
@@ -504,7 +634,7 @@ int llms_attend_composed_mfma(void* out, int out_stride, const void* q, int q_st
     a.upk = upk, a.tok = upk * a.tpw, a.kv_per_wg = 1, a.units = upk;
     a.slices = upk == 1 ? 4 : 1;
     a.blocks_per_seq = (max_new + a.tok - 1) / a.tok;
-    const size_t lds = a.slices > 1 ? (size_t)a.units * a.slices * maps * 16 * (2 + dv) * sizeof(float) : 0;
+    const size_t lds = ((a.slices > 1 ? (size_t)a.units * a.slices * maps * 16 * (2 + dv) : 0) + AM_PAGE_CACHE) * sizeof(float);
     dim3 grid(n_seqs * a.blocks_per_seq, kv_heads);
     LLMS_REQUIRE(grid.y <= 65535, "attend_composed_mfma: too many key/value heads");
     if (maps == 2) return launch<2, false, 1, 256>(a, grid, upk * a.slices * LLMS_WAVE, lds, stream);

@@ -19,6 +19,79 @@ __global__ __launch_bounds__(S32_THREADS) void embed_scale_kernel(float* __restr
     for (int c = threadIdx.x; c < hidden; c += S32_THREADS) out[(size_t)n * hidden + c] = to_f32(row[c]) * scale;
 }
 
+// Rows whose length is a multiple of 4: a thread brings up to S32_VEC float4 of its row at once (rows of up to
+// 4 * S32_VEC * S32_THREADS), so a row costs one wait for memory and not one per 256 elements.
+#define S32_VEC 8
+
+template <typename T>
+__global__ __launch_bounds__(S32_THREADS) void rmsnorm32_vec_kernel(T* __restrict__ out, const float* __restrict__ x,
+                                                                    const float* __restrict__ weight,
+                                                                    const int* __restrict__ rows, int hidden, float eps,
+                                                                    float offset) {
+    __shared__ float lds[16];
+    const int r = blockIdx.x;
+    const float4* xr = reinterpret_cast<const float4*>(x + (size_t)(rows ? rows[r] : r) * hidden);
+    const float4* wr = reinterpret_cast<const float4*>(weight);
+    const int n4 = hidden / 4;
+    float4 v[S32_VEC], w[S32_VEC];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < S32_VEC; ++i) {
+        const int c = threadIdx.x + i * S32_THREADS;
+        v[i] = c < n4 ? xr[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+        w[i] = c < n4 ? wr[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+#pragma unroll
+    for (int i = 0; i < S32_VEC; ++i) ss += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
+    const float inv = 1.0f / sqrtf(block_sum(ss, lds) / (float)hidden + eps);
+    T* orow = out + (size_t)r * hidden;
+#pragma unroll
+    for (int i = 0; i < S32_VEC; ++i) {
+        const int c = threadIdx.x + i * S32_THREADS;
+        if (c < n4) {
+            orow[4 * c + 0] = from_f32<T>(v[i].x * inv * (offset + w[i].x));
+            orow[4 * c + 1] = from_f32<T>(v[i].y * inv * (offset + w[i].y));
+            orow[4 * c + 2] = from_f32<T>(v[i].z * inv * (offset + w[i].z));
+            orow[4 * c + 3] = from_f32<T>(v[i].w * inv * (offset + w[i].w));
+        }
+    }
+}
+
+__device__ __forceinline__ float4 gate4(float4 z, float4 b) {
+    return make_float4(1.f / (1.f + expf(-(z.x + b.x))), 1.f / (1.f + expf(-(z.y + b.y))), 1.f / (1.f + expf(-(z.z + b.z))),
+                       1.f / (1.f + expf(-(z.w + b.w))));
+}
+
+// gated_add for rows of a multiple of 4 (and gate columns at multiples of 4): grid (rows, ceil(hidden / 4 / threads))
+__global__ __launch_bounds__(S32_THREADS) void gated_add_vec_kernel(float* __restrict__ x, const float* __restrict__ z,
+                                                                    int z_stride, int z_col0, int z_col1,
+                                                                    const float* __restrict__ bias0,
+                                                                    const float* __restrict__ bias1,
+                                                                    const float* __restrict__ y0, int y0_stride,
+                                                                    const float* __restrict__ y1, int y1_stride,
+                                                                    int hidden) {
+    const int n = blockIdx.x, c = 4 * (blockIdx.y * S32_THREADS + threadIdx.x);
+    if (c >= hidden) return;
+    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f), one = make_float4(1.f, 1.f, 1.f, 1.f);
+    auto at = [](const float* p) { return *reinterpret_cast<const float4*>(p); };
+    // every load is asked for before the first is used
+    const float4 xv = at(x + (size_t)n * hidden + c);
+    const float4 a0 = y0 ? at(y0 + (size_t)n * y0_stride + c) : zero;
+    const float4 a1 = y1 ? at(y1 + (size_t)n * y1_stride + c) : zero;
+    const float4 z0 = (y0 && z_col0 >= 0) ? at(z + (size_t)n * z_stride + z_col0 + c) : zero;
+    const float4 z1 = (y1 && z_col1 >= 0) ? at(z + (size_t)n * z_stride + z_col1 + c) : zero;
+    const float4 b0 = (y0 && z_col0 >= 0 && bias0) ? at(bias0 + c) : zero;
+    const float4 b1 = (y1 && z_col1 >= 0 && bias1) ? at(bias1 + c) : zero;
+    const float4 g0 = (y0 && z_col0 >= 0) ? gate4(z0, b0) : one;
+    const float4 g1 = (y1 && z_col1 >= 0) ? gate4(z1, b1) : one;
+    float4 r;
+    r.x = xv.x + (g0.x * a0.x + g1.x * a1.x);
+    r.y = xv.y + (g0.y * a0.y + g1.y * a1.y);
+    r.z = xv.z + (g0.z * a0.z + g1.z * a1.z);
+    r.w = xv.w + (g0.w * a0.w + g1.w * a1.w);
+    *reinterpret_cast<float4*>(x + (size_t)n * hidden + c) = r;
+}
+
 template <typename T>
 __global__ __launch_bounds__(S32_THREADS) void rmsnorm32_kernel(T* __restrict__ out, const float* __restrict__ x,
                                                                 const float* __restrict__ weight,
@@ -79,6 +152,14 @@ int llms_embed_scale(int dtype, float* out, const void* table, const int* ids, i
 int llms_rmsnorm32(int dtype, void* out, const float* x, const float* weight, const int* rows, float eps, float offset,
                    int n_out, int hidden, hipStream_t stream) {
     LLMS_REQUIRE(n_out > 0 && hidden > 0, "rmsnorm32: sizes must be positive");
+    LLMS_REQUIRE(dtype == 0 || dtype == 1, "rmsnorm32: dtype must be 0 (float32) or 1 (bfloat16)");
+    if (hidden % 4 == 0 && hidden <= 4 * S32_VEC * S32_THREADS && ((uintptr_t)x % 16) == 0 && ((uintptr_t)weight % 16) == 0) {
+        if (dtype == 0)
+            rmsnorm32_vec_kernel<float><<<n_out, S32_THREADS, 0, stream>>>((float*)out, x, weight, rows, hidden, eps, offset);
+        else
+            rmsnorm32_vec_kernel<bf16><<<n_out, S32_THREADS, 0, stream>>>((bf16*)out, x, weight, rows, hidden, eps, offset);
+        LLMS_LAUNCH_CHECK();
+    }
     if (dtype == 0)
         rmsnorm32_kernel<float><<<n_out, S32_THREADS, 0, stream>>>((float*)out, x, weight, rows, hidden, eps, offset);
     else if (dtype == 1)
@@ -94,8 +175,18 @@ int llms_gated_add(float* x, const float* z, int z_stride, int z_col0, int z_col
     LLMS_REQUIRE(n > 0 && hidden > 0, "gated_add: sizes must be positive");
     LLMS_REQUIRE(y0 || y1, "gated_add: no branch to add");
     LLMS_REQUIRE(z || (z_col0 < 0 && z_col1 < 0), "gated_add: gate columns named without gate products");
-    gated_add_kernel<<<n, S32_THREADS, 0, stream>>>(x, z, z_stride, z_col0, z_col1, bias0, bias1, y0, y0_stride, y1,
-                                                    y1_stride, hidden);
+    auto aligned = [](const void* p) { return ((uintptr_t)p % 16) == 0; };
+    const bool vec = hidden % 4 == 0 && z_stride % 4 == 0 && y0_stride % 4 == 0 && y1_stride % 4 == 0 &&
+                     (z_col0 < 0 || z_col0 % 4 == 0) && (z_col1 < 0 || z_col1 % 4 == 0) && aligned(x) && aligned(z) &&
+                     aligned(bias0) && aligned(bias1) && aligned(y0) && aligned(y1);
+    if (vec) {
+        dim3 grid(n, (hidden / 4 + S32_THREADS - 1) / S32_THREADS);
+        gated_add_vec_kernel<<<grid, S32_THREADS, 0, stream>>>(x, z, z_stride, z_col0, z_col1, bias0, bias1, y0, y0_stride,
+                                                               y1, y1_stride, hidden);
+    } else {
+        gated_add_kernel<<<n, S32_THREADS, 0, stream>>>(x, z, z_stride, z_col0, z_col1, bias0, bias1, y0, y0_stride, y1,
+                                                        y1_stride, hidden);
+    }
     LLMS_LAUNCH_CHECK();
 }
 

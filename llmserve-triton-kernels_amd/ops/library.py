@@ -977,11 +977,13 @@ def attend_composed_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tenso
                          block_size: int, scale: float, maps: int = 1, window: int = 0, keep_first: int = 0,
                          chunk: int = 0, slopes: torch.Tensor | None = None, talk: torch.Tensor | None = None,
                          lam: float = 0.0, head_norm: bool = False, eps: float = 0.0, out_scale: float = 1.0,
-                         table_rows: torch.Tensor | None = None) -> torch.Tensor:
+                         table_rows: torch.Tensor | None = None, shares: int = 1) -> torch.Tensor:
     """`attend_composed` on the matrix cores (bfloat16) for requests [seq_begin, seq_begin + n_seqs) of a step: request
     b owns rows cu_seqlens[b] .. cu_seqlens[b+1] of q and out, brings at most `max_new` tokens and is context_lens[b]
     long after the step (0: padding, left alone).  Same arguments and arithmetic otherwise; the weights are rounded
-    to bfloat16 as the operand of the value product."""
+    to bfloat16 as the operand of the value product.  `shares` > 1 (requests of one token whose heads' weights are
+    mixed): every request's keys are shared out to that many workgroups in two launches (maxima and sums; weights
+    and values), their 32-bit parts added up by a third."""
     dev = _dev(out, q, k_pool, v_pool, block_tables, cu_seqlens, context_lens, slopes, talk, table_rows)
     if not attend_composed_mfma_supported(q.dtype, heads, kv_heads, dk, dv, block_size, talk is not None):
         raise ValueError("attend_composed_mfma does not take these sizes; see attend_composed_mfma_supported")
@@ -1016,12 +1018,20 @@ def attend_composed_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tenso
         _f32(talk, "talk", heads * heads)
     if n_seqs == 0 or max_new <= 0 or q.shape[0] == 0:
         return out
+    ws_stats = ws_o = None
+    if not (shares > 1 and talk is not None and max_new == 1):
+        shares = 1
+    else:
+        shares = min(int(shares), 64)
+        ws_stats = torch.empty((q.shape[0], heads, shares, 2), dtype=torch.float32, device=dev)
+        ws_o = torch.empty((shares, q.shape[0], heads * dv), dtype=torch.float32, device=dev)
     _check(load("attention_composed_mfma").llms_attend_composed_mfma(
         _ptr(out), c_int(out.stride(0)), _ptr(q), c_int(q.stride(0)), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables),
         _ptr(table_rows), c_int(block_tables.shape[1]), _ptr(cu_seqlens), _ptr(context_lens), c_int(seq_begin),
         c_int(n_seqs), c_int(max_new), c_int(heads), c_int(kv_heads), c_int(maps), c_int(dk), c_int(dv),
         c_int(block_size), c_int(window), c_int(keep_first), c_int(chunk), c_float(scale), _ptr(slopes), _ptr(talk),
-        c_float(lam), c_int(1 if head_norm else 0), c_float(eps), c_float(out_scale), _stream(dev)),
+        c_float(lam), c_int(1 if head_norm else 0), c_float(eps), c_float(out_scale), c_int(shares), _ptr(ws_stats),
+        _ptr(ws_o), c_int(q.shape[0]), _stream(dev)),
         "attend_composed_mfma")
     return out
 

@@ -175,6 +175,18 @@ class ComposedAttention(Mixer):
         args = (out, q, paged.k_pool, paged.v_pool, view.block_tables, batch.cu_seqlens, batch.context_lens)
         n_dec = batch.num_decode
         if n_dec:
-            ops.attend_composed_mfma(*args, 0, n_dec, 1, **common)
+            ops.attend_composed_mfma(*args, 0, n_dec, 1, shares=self.decode_shares(n_dec, batch.max_decode_context,
+                                                                                  ops.compute_units(q.device)), **common)
         if n_dec < batch.num_seqs:
             ops.attend_composed_mfma(*args, n_dec, batch.num_seqs - n_dec, batch.max_count, **common)
+
+    def decode_shares(self, n_requests: int, max_context: int, cus: int = 256) -> int:
+        """Workgroups that share the keys of one decoding request when the heads' weights are mixed.  Such a request is
+        one workgroup (all its heads must meet for the mixing), which alone keeps one compute unit busy for as long
+        as its keys last; while the batch leaves compute units idle its keys go to several, 128 keys a share at
+        least, at the price of two more launches."""
+        if not self.talking:
+            return 1
+        reach = min(x for x in (max_context, self.chunk, None if self.window is None else self.window + self.keep_first)
+                    if x is not None)
+        return max(1, min(8, cus // max(n_requests, 1), int(reach) // 128))

@@ -34,7 +34,8 @@ def close(got, ref, dtype, what=""):
 
 # ------------------------------------------------------------------------------ the 32-bit stream's kernels
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_scaled_embedding_norm_and_gated_sum(dtype):
+@pytest.mark.parametrize("hidden", [100, 98, 2048])  # rows of a multiple of 4 go to the kernels that read 16 bytes a thread
+def test_scaled_embedding_norm_and_gated_sum(dtype, hidden):
     from llmserve.ops import library as ops
 
     table = rnd(50, 72, seed=1).to(dtype)
@@ -42,22 +43,25 @@ def test_scaled_embedding_norm_and_gated_sum(dtype):
     x = ops.embed_scale(torch.empty(4, 72, device=DEV), table.to(DEV), ids.to(DEV), 1.7)
     close(x, table.double()[ids.long()] * 1.7, torch.float32, "embedding")
 
-    stream = rnd(6, 100, seed=2).float()
-    w = rnd(100, seed=3, scale=0.2).float()
-    out = ops.rmsnorm32(torch.empty(6, 100, dtype=dtype, device=DEV), stream.to(DEV), w.to(DEV), 1e-5, 1.0)
+    stream = rnd(6, hidden, seed=2).float()
+    w = rnd(hidden, seed=3, scale=0.2).float()
+    out = ops.rmsnorm32(torch.empty(6, hidden, dtype=dtype, device=DEV), stream.to(DEV), w.to(DEV), 1e-5, 1.0)
     close(out, pd.norm_zero_centred(stream.double(), w.double(), 1e-5), dtype, "norm")
     rows = torch.tensor([4, 0], dtype=torch.int32, device=DEV)
-    out = ops.rmsnorm32(torch.empty(2, 100, dtype=dtype, device=DEV), stream.to(DEV), w.to(DEV), 1e-5, 1.0, rows=rows)
+    out = ops.rmsnorm32(torch.empty(2, hidden, dtype=dtype, device=DEV), stream.to(DEV), w.to(DEV), 1e-5, 1.0, rows=rows)
     close(out, pd.norm_zero_centred(stream.double(), w.double(), 1e-5)[[4, 0]], dtype, "norm of rows")
 
-    z, a, f = rnd(6, 200, seed=4).float(), rnd(6, 100, seed=5).float(), rnd(6, 100, seed=6).float()
-    b1, b2 = rnd(100, seed=7).float(), rnd(100, seed=8).float()
-    ref = stream.double() + torch.sigmoid(z[:, :100].double() + b1.double()) * a.double() \
-        + torch.sigmoid(z[:, 100:].double() + b2.double()) * f.double()
-    got = ops.gated_add(stream.clone().to(DEV), [(a.to(DEV), 0, b1.to(DEV)), (f.to(DEV), 100, b2.to(DEV))], z.to(DEV))
+    z, a, f = rnd(6, 2 * hidden, seed=4).float(), rnd(6, hidden, seed=5).float(), rnd(6, hidden, seed=6).float()
+    b1, b2 = rnd(hidden, seed=7).float(), rnd(hidden, seed=8).float()
+    ref = stream.double() + torch.sigmoid(z[:, :hidden].double() + b1.double()) * a.double() \
+        + torch.sigmoid(z[:, hidden:].double() + b2.double()) * f.double()
+    got = ops.gated_add(stream.clone().to(DEV), [(a.to(DEV), 0, b1.to(DEV)), (f.to(DEV), hidden, b2.to(DEV))], z.to(DEV))
     close(got, ref, torch.float32, "two gated branches")
     got = ops.gated_add(stream.clone().to(DEV), [(a.to(DEV), None, None)])
     close(got, stream.double() + a.double(), torch.float32, "one branch without a gate")
+    ref = stream.double() + a.double() + torch.sigmoid(z[:, hidden:].double() + b2.double()) * f.double()
+    got = ops.gated_add(stream.clone().to(DEV), [(a.to(DEV), None, None), (f.to(DEV), hidden, b2.to(DEV))], z.to(DEV))
+    close(got, ref, torch.float32, "a plain branch beside a gated one")
 
 
 # ------------------------------------------------------------------------------ convolution, state and cache store
@@ -250,7 +254,7 @@ def test_a_key_that_stands_out_shows_every_edge():
 
 
 # ------------------------------------------------------------------------------ the matrix-core kernel
-def attend_mfma(seqs, bs, **kw):
+def attend_mfma(seqs, bs, shares=1, **kw):
     """`seqs`: per request (q [t, S, dk], k, v, first new row, number of new rows); requests that bring one row
     first.  All share one pool.  Returns the kernel's rows per request."""
     from llmserve.ops import library as ops
@@ -277,7 +281,7 @@ def attend_mfma(seqs, bs, **kw):
     args = (out, qs, k_pool, v_pool, table, as_i32(cu), as_i32([a + n for *_x, a, n in seqs]))
     common = dict(dk=seqs[0][0].shape[2], dv=dv, block_size=bs, table_rows=as_i32(rows_of), **kw)
     if n_dec:
-        ops.attend_composed_mfma(*args, 0, n_dec, 1, **common)
+        ops.attend_composed_mfma(*args, 0, n_dec, 1, shares=shares, **common)
     if n_dec < len(seqs):
         ops.attend_composed_mfma(*args, n_dec, len(seqs) - n_dec, max(n for *_x, n in seqs), **common)
     return [out[cu[i]: cu[i + 1]] for i in range(len(seqs))]
@@ -334,6 +338,12 @@ def test_matrix_core_kernel_mixed_heads(heads, kv, dk, dv, chunk, bs):
                       talk=talk.float().to(DEV))
     for i, (g, r) in enumerate(zip(got, refs)):
         close(g, r, dt, f"request {i}")
+    # the keys of the requests of one token shared out to several workgroups
+    for shares in (2, 5):
+        got = attend_mfma(seqs[:2], bs, shares=shares, heads=heads, kv_heads=kv, chunk=chunk or 0, scale=0.3,
+                          slopes=slopes.float().to(DEV), talk=talk.float().to(DEV))
+        for i, (g, r) in enumerate(zip(got, refs[:2])):
+            close(g, r, dt, f"request {i} in {shares} shares")
     got = attend_mfma(seqs[2:3], bs, heads=heads, kv_heads=kv, chunk=chunk or 0, scale=0.3)  # neither slopes nor mixing
     ref = pd.talking_heads(seqs[2][0].double(), seqs[2][1].double(), seqs[2][2].double(), pd.visible_chunk(90, chunk), 0.3,
                            None, None)
