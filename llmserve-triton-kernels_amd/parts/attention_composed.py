@@ -139,11 +139,22 @@ class ComposedAttention(Mixer):
             self.lam = math.exp(dot[0]) - math.exp(dot[1]) + self.diff
 
     # ---- one step ------------------------------------------------------------------------------------
-    def forward(self, x, batch, cache):
+    @property
+    def input_weight(self):
+        """The stacked q, k, v projection: an arrangement may fold it into a product of its own (32-bit result) and
+        hand the result back as `projected`."""
+        return self.qkv_weight
+
+    @input_weight.setter
+    def input_weight(self, weight):
+        self.qkv_weight = weight
+
+    def forward(self, x, batch, cache, projected=None):
         paged, state = cache if isinstance(cache, tuple) else (cache, None)
         view = batch.groups[paged.group_id]
         heads, kv, dk, dv = self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim
-        proj = linear(x, self.qkv_weight, out_dtype=torch.float32)  # q, k and v side by side, unrounded
+        # q, k and v side by side, unrounded
+        proj = projected if projected is not None else linear(x, self.qkv_weight, out_dtype=torch.float32)
         q = torch.empty((proj.shape[0], self.cq), dtype=x.dtype, device=x.device)
         conv, taps = self.taps > 1, self.taps > 0  # (one tap is a factor per channel and needs no state)
         ops.conv_store(q, proj, cq=self.cq, k_heads=kv * self.maps, dk=dk, v_heads=kv, dv=dv,

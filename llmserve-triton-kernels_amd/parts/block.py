@@ -47,28 +47,52 @@ class ParallelBlock(Block):
 
     def __init__(self, parts):
         super().__init__(parts)
-        self._stacked = None  # the two gates' weights as one matrix, made at the first step
+        self._stacked = None  # the gates' weights (and the mixer's input projection) as one matrix, made at the first step
+        self._mixer_columns = None
 
-    def _gate_products(self, h):
-        """(products [N, columns] or None, column of the mixer's gate or None, column of the feed-forward's)."""
+    def _stack(self):
+        """One matrix for every product of h whose result stays 32-bit: the two gates, and the mixer's input
+        projection where the mixer offers it (`input_weight`, taken back as `projected`).  The parts' own
+        weights become views of it, so nothing is held twice."""
         gm, gf = self.mixer_gate, self.feed_forward_gate
         wm, wf = gm.weight, gf.weight
-        if wm is not None and wf is not None:  # one product for both
-            if self._stacked is None:
-                self._stacked = torch.cat([wm, wf], dim=0).contiguous()
-            return linear(h, self._stacked, out_dtype=torch.float32), 0, wm.shape[0]
+        if wm is None or wf is None:
+            return False
+        if self._stacked is None:
+            pieces = [wm, wf]
+            mixer_w = getattr(self.mixer, "input_weight", None)
+            if mixer_w is not None and mixer_w.dtype == wm.dtype and mixer_w.shape[1] == wm.shape[1]:
+                pieces.append(mixer_w)
+            self._stacked = torch.cat(pieces, dim=0).contiguous()
+            a, b = wm.shape[0], wm.shape[0] + wf.shape[0]
+            gm.weight, gf.weight = self._stacked[:a], self._stacked[a:b]
+            if len(pieces) == 3:
+                self.mixer.input_weight = self._stacked[b:]
+                self._mixer_columns = (b, self._stacked.shape[0])
+        return True
+
+    def _gate_products(self, h):
+        """(products [N, columns] or None, column of the mixer's gate or None, column of the feed-forward's,
+        the mixer's projected input or None)."""
+        gm, gf = self.mixer_gate, self.feed_forward_gate
+        if self._stack():  # one product for all
+            out = linear(h, self._stacked, out_dtype=torch.float32)
+            projected = None
+            if self._mixer_columns is not None:
+                projected = out[:, self._mixer_columns[0]: self._mixer_columns[1]]
+            return out, 0, gm.weight.shape[0], projected
         zm, zf = gm.products(h), gf.products(h)
         if zm is not None and zf is not None:
-            return torch.cat([zm, zf], dim=1), 0, zm.shape[1]
+            return torch.cat([zm, zf], dim=1), 0, zm.shape[1], None
         one = zm if zm is not None else zf
-        return one, (0 if zm is not None else None), (0 if zf is not None else None)
+        return one, (0 if zm is not None else None), (0 if zf is not None else None), None
 
     def forward(self, x, delta, batch, cache):
         if delta is not None or x.dtype != torch.float32:
             raise ValueError("the parallel arrangement keeps a closed 32-bit residual stream")
         h = self.norm.forward(x)
-        z, col_m, col_f = self._gate_products(h)
-        a = self.mixer.forward(h, batch, cache)
+        z, col_m, col_f, projected = self._gate_products(h)
+        a = self.mixer.forward(h, batch, cache) if projected is None else self.mixer.forward(h, batch, cache, projected=projected)
         f = self.feed_forward.forward(h)
         branches = []
         for y, col, gate in ((a, col_m, self.mixer_gate), (f, col_f, self.feed_forward_gate)):

@@ -162,6 +162,10 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
+    """A mixer may offer `input_weight` ([columns, hidden], settable: the arrangement may replace it by a view of a
+    larger matrix) and then takes `forward(x, batch, cache, projected=...)`: the 32-bit product x input_weight^T that
+    the arrangement formed together with products of its own."""
+
     accepts_deferred_norm = False
 
     def cache_spec(self) -> PagedCacheSpec | StateCacheSpec | None:
