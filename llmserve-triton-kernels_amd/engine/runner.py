@@ -101,10 +101,10 @@ class ModelRunner:
         engine_config = engine_config or EngineConfig()
         engine_config.validate()
         device = cls._device(device)
-        ops.ensure_built(engine_config.dtype)
         arch, config, _raw = read_config(model_dir)
         dtype = _TORCH_DTYPES[engine_config.dtype]
         model = Model(arch.build_spec(config), BuildContext(dtype, device))
+        ops.ensure_built(engine_config.dtype, extra=model.libraries(engine_config.dtype))
         infos = model.param_infos()
         ignore = {model.spec.weights["head"] + "weight"} if getattr(model.head, "tied", False) else set()
         ignore |= set(model.spec.unused_tensors)
@@ -120,11 +120,11 @@ class ModelRunner:
         engine_config = engine_config or EngineConfig()
         engine_config.validate()
         device = cls._device(device)
-        ops.ensure_built(engine_config.dtype)
         arch = architecture_of(config_dict)
         config = arch.config_class.from_dict(config_dict)
         dtype = _TORCH_DTYPES[engine_config.dtype]
         model = Model(arch.build_spec(config), BuildContext(dtype, device))
+        ops.ensure_built(engine_config.dtype, extra=model.libraries(engine_config.dtype))
         tensors = random_tensors(model.param_infos(), seed, dtype, device if on_device else "cpu")
         model.load({k: v.to(device) for k, v in tensors.items()})
         return cls(model, config, engine_config, device)

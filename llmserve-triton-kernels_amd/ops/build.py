@@ -37,11 +37,17 @@ HIPCC_FLAGS = [
     "-Wno-unused-result", "-Wno-unknown-warning-option", "-Wno-pass-failed",
 ]
 
-# Which libraries the step function of a model of a given dtype needs (the sampler's library is
-# built when something is first sampled).
+# Which libraries the step function of every model of a given dtype needs: the products and the elementwise
+# kernels.  Parts add their own (`Part.libraries`: an attention its kernels, a 32-bit stream its own), so a model
+# compiles what it runs and no more; the sampler's library is built when something is first sampled.
+BASE = {
+    "float32": ("elementwise", "gemm"),
+    "bfloat16": ("elementwise", "gemm", "gemm_stream", "gemm_decode"),
+}
+# (everything the built-in parts of the Llama decoder load: what `ensure_built(dtype)` without a model builds)
 GROUPS = {
-    "float32": ("elementwise", "gemm", "attention"),
-    "bfloat16": ("elementwise", "gemm", "attention", "gemm_stream", "gemm_decode", "attention_mfma"),
+    "float32": BASE["float32"] + ("attention",),
+    "bfloat16": BASE["bfloat16"] + ("attention", "attention_mfma"),
 }
 
 

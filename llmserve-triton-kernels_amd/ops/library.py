@@ -46,9 +46,10 @@ def load(name: str) -> ctypes.CDLL:
         return lib
 
 
-def ensure_built(dtype_name: str, verbose: bool = True) -> None:
-    """Compile (if missing) and load every library a model of this dtype uses."""
-    names = _build.GROUPS[dtype_name]
+def ensure_built(dtype_name: str, verbose: bool = True, extra=None) -> None:
+    """Compile (if missing, side by side) and load the libraries a model of this dtype uses: with `extra` (what the
+    model's parts name) the products and elementwise kernels and those; without, the Llama decoder's."""
+    names = _build.GROUPS[dtype_name] if extra is None else tuple(dict.fromkeys(_build.BASE[dtype_name] + tuple(extra)))
     _build.build(names, verbose=verbose)
     for n in names:
         load(n)

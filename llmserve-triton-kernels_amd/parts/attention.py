@@ -47,6 +47,9 @@ class Attention(Mixer):
     def cache_spec(self):
         return PagedCacheSpec(self.num_kv_heads, self.head_dim, self.window)
 
+    def libraries(self, dtype_name):
+        return ("attention", "attention_mfma") if dtype_name == "bfloat16" else ("attention",)
+
     def param_infos(self):
         h, d = self.hidden, self.head_dim
         infos = {"q_proj.weight": ParamInfo((self.num_heads * d, h)),

@@ -96,6 +96,9 @@ class ComposedAttention(Mixer):
         self.qkv_weight = self.o_weight = self.taps_w = self.talk = self.slopes = None
         self.lam = 0.0
 
+    def libraries(self, dtype_name):
+        return ("attention_composed", "attention_composed_mfma") if dtype_name == "bfloat16" else ("attention_composed",)
+
     # ---- what it keeps between steps -------------------------------------------------------------
     def cache_spec(self):
         paged = PagedCacheSpec(num_kv_heads=self.num_kv_heads * self.maps, head_dim=self.head_dim,

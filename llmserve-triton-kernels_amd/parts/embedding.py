@@ -34,6 +34,9 @@ class TokenEmbedding(Part):
     def param_infos(self):
         return {self.tensor: ParamInfo((self.vocab, self.hidden))}
 
+    def libraries(self, dtype_name):
+        return ("stream32",) if self.stream == "float32" else ()
+
     def load(self, tensors):
         self.weight = tensors[self.tensor].contiguous()
 

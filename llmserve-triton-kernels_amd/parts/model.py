@@ -61,6 +61,14 @@ class Model:
         if getattr(self.head, "tied", False):
             self.head.load({"weight": self.embedding.weight})
 
+    def libraries(self, dtype_name: str) -> tuple[str, ...]:
+        """Kernel libraries the model's parts name, in first-use order without repeats."""
+        names: dict[str, None] = {}
+        for _, part in self._parts():
+            for name in part.libraries(dtype_name):
+                names[name] = None
+        return tuple(names)
+
     def graph_safe(self) -> bool:
         """Whether a decode-only step through this model may be captured as a HIP graph."""
         parts = [part for _, part in self._parts()]

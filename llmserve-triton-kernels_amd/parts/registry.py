@@ -58,6 +58,11 @@ class Part:
     def param_infos(self) -> dict[str, ParamInfo]:
         return {}
 
+    def libraries(self, dtype_name: str) -> tuple[str, ...]:
+        """Kernel libraries (names of ``csrc/*.hip``) this part loads beside the products' and the elementwise
+        kernels', for an engine of the given dtype: they are compiled before the first step."""
+        return ()
+
     def load(self, tensors: dict[str, torch.Tensor]) -> None:
         """Take the part's tensors (already on the device, in their stored dtype) and set up
         device constants.  Called once, also for parts without tensors."""

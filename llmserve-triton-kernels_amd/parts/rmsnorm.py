@@ -68,6 +68,9 @@ class RMSNorm32(Norm):
     def param_infos(self):
         return {self.tensor: ParamInfo((self.hidden,), "around_zero" if self.offset else "norm")}
 
+    def libraries(self, dtype_name):
+        return ("stream32",)
+
     def load(self, tensors):
         self.weight = tensors[self.tensor].float().contiguous()
 
