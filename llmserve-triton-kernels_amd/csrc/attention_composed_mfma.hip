@@ -421,7 +421,7 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
         // second walk: normalised weights through LDS, mixed, times the values
         for (int round = 0; round < n_rounds; ++round) {
             const int group = (round * NS + slice) * NSG + share;
-            const bool some = group < n_groups;  // (a slice without keys in this round only keeps the barriers' count)
+            const bool some = group < n_groups;  // (a slice without keys at this turn of the loop only keeps the barriers' count)
             s16x4 vf[MAXU][TG][MAXTV];
 #pragma unroll
             for (int uu = 0; uu < MAXU; ++uu) {
