@@ -632,13 +632,15 @@ int llms_attend_composed_mfma(void* out, int out_stride, const void* q, int q_st
     int upk = 4;
     while (upk > 1 && (upk - 1) * a.tpw >= max_new) --upk;
     a.upk = upk, a.tok = upk * a.tpw, a.kv_per_wg = 1, a.units = upk;
-    a.slices = upk == 1 ? 4 : 1;
+    a.slices = 1;
+    if (upk == 1)  // few tokens (decoding): the groups of keys go to 8 waves, or to 4 where 8 would not fit the LDS
+        a.slices = ((size_t)8 * maps * 16 * (2 + dv) + AM_PAGE_CACHE) * sizeof(float) <= 96 * 1024 ? 8 : 4;
     a.blocks_per_seq = (max_new + a.tok - 1) / a.tok;
     const size_t lds = ((a.slices > 1 ? (size_t)a.units * a.slices * maps * 16 * (2 + dv) : 0) + AM_PAGE_CACHE) * sizeof(float);
     dim3 grid(n_seqs * a.blocks_per_seq, kv_heads);
     LLMS_REQUIRE(grid.y <= 65535, "attend_composed_mfma: too many key/value heads");
-    if (maps == 2) return launch<2, false, 1, 256>(a, grid, upk * a.slices * LLMS_WAVE, lds, stream);
-    return launch<1, false, 1, 256>(a, grid, upk * a.slices * LLMS_WAVE, lds, stream);
+    if (maps == 2) return launch<2, false, 1, 512>(a, grid, upk * a.slices * LLMS_WAVE, lds, stream);
+    return launch<1, false, 1, 512>(a, grid, upk * a.slices * LLMS_WAVE, lds, stream);
 }
 
 }  // extern "C"

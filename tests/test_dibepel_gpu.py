@@ -212,7 +212,7 @@ def test_a_key_that_stands_out_shows_every_edge():
     """One key is made to carry nearly all the weight of one query; its value is a marker.  Just inside a window, a
     chunk or the kept first tokens the marker must come out, just outside it must be gone; also far back, and where
     the key lies on a page's border."""
-    t, dk, dv, bs = 300, 16, 8, 16
+    t, dk, dv, bs = 300, 16, 16, 16
     g = torch.Generator().manual_seed(5)
     q = torch.randn(t, 1, dk, generator=g, dtype=F64)
     k = torch.randn(t, 1, dk, generator=g, dtype=F64)
@@ -225,9 +225,16 @@ def test_a_key_that_stands_out_shows_every_edge():
         return kk, vv
 
     def marker_seen(i, j, **kw):
+        """By the kernel for any size (32-bit, the query alone) and by the matrix-core kernel (bfloat16), there both as
+        a request's only new token and as the last token of a whole prompt: all three must agree."""
         kk, vv = marked(i, j)
         out = attend(q, kk, vv, torch.float32, bs, rows=[i], heads=1, kv_heads=1, scale=dk ** -0.5, **kw)
-        return float(out[0, 0]) > 3.5
+        seen = float(out[0, 0]) > 3.5
+        cut = (q[: i + 1], kk[: i + 1], vv[: i + 1])
+        decoded = attend_mfma([(*cut, i, 1)], bs, heads=1, kv_heads=1, scale=dk ** -0.5, **kw)[0]
+        prompt = attend_mfma([(*cut, 0, i + 1)], bs, heads=1, kv_heads=1, scale=dk ** -0.5, **kw)[0]
+        assert (float(decoded[0, 0]) > 3.5) == seen and (float(prompt[-1, 0]) > 3.5) == seen, (i, j, kw)
+        return seen
 
     window, keep, chunk = 40, 20, 64
     for i in (40, 63, 64, 200, 299):
@@ -292,6 +299,7 @@ MFMA_DIFF = [  # heads, kv_heads, dk, dv, window, keep_first, block size
     (4, 4, 16, 48, 40, 20, 16),
     (16, 2, 64, 128, 33, 0, 16),
     (3, 1, 16, 16, None, 0, 4),  # three heads in a unit of 16 columns: five tokens and a padded column
+    (16, 1, 16, 32, 21, 3, 8),  # sixteen heads on one key/value head: a unit is one token
 ]
 
 
@@ -319,6 +327,8 @@ MFMA_TALK = [  # heads, kv_heads, dk, dv, chunk, block size
     (32, 4, 64, 64, 128, 16),
     (32, 32, 32, 128, None, 16),  # two units a wave
     (6, 2, 16, 16, 50, 4),
+    (16, 1, 32, 16, 40, 8),  # a unit is one token
+    (24, 24, 16, 16, 30, 16),  # 24 units in 12 waves
 ]
 
 
