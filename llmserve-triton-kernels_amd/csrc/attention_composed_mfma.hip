@@ -29,6 +29,8 @@
 // were given back (table entry < 0) and values behind the request's end are read as zeros.
 #include "common.h"
 
+#include <type_traits>
+
 #define AM_PAGE_CACHE 1024  // page ids (4 bytes each) a workgroup keeps in LDS
 
 #define LOG2E 1.4426950408889634f
@@ -49,7 +51,7 @@ struct MfmaArgs {
     const float* slopes;
     const float* talk;
     int out_stride, q_stride, max_blocks;
-    int seq_begin, blocks_per_seq;
+    int seq_begin, n_seqs, blocks_per_seq;
     int heads, kv_heads, grp, dk, dv, block_size;
     int window, keep_first, chunk;
     int tok, tpw, upk, units, kv_per_wg, slices;
@@ -92,7 +94,9 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
     const int wave = threadIdx.x / LLMS_WAVE, lane = threadIdx.x % LLMS_WAVE, nwaves = blockDim.x / LLMS_WAVE;
     const int col = lane % 16, q4 = lane / 16;
     const int NS = a.slices, slice = wave % NS, uw = wave / NS, n_uw = nwaves / NS;
-    const int b = a.seq_begin + blockIdx.x / a.blocks_per_seq, blk = blockIdx.x % a.blocks_per_seq;
+    // blocks of tokens are handed out from every request's end: the last block sees the most keys and should not
+    // be the last to start
+    const int b = a.seq_begin + blockIdx.x % a.n_seqs, blk = a.blocks_per_seq - 1 - blockIdx.x / a.n_seqs;
     const int row0 = a.cu_seqlens[b], count = a.cu_seqlens[b + 1] - row0;
     const int end = a.context_lens[b];
     const int t0 = blk * a.tok;
@@ -170,9 +174,32 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
     // v_exp_f32; a maximum of -inf (nothing seen yet) is replaced by a large negative number, so that exp2(-inf - m) is 0
     const float scale2 = a.scale * LOG2E;
     const size_t k_page = (size_t)G * MAPS * bs * dk, v_page = (size_t)G * dv * bs;  // elements in a page
-    auto scores = [&](int uu, int m, int group, float sc[TG][4]) {
+    // A group is *plain* when pages hold a multiple of 16 keys, keys and values are as wide as the kernel's tiles, and
+    // all its keys are there, on pages whose ids are in LDS: then a tile's page and place are the same for every
+    // lane, worked out by the scalar unit, and a lane adds only its own fixed offset.
+    auto plain_group = [&](int group) {
+        if constexpr (TALK) return false;  // (with mixed heads the second set of loops did not fit the 128 registers of 16 waves)
+        const int last = tile_start(group * TG + TG - 1) + 15;
+        return (bs & 15) == 0 && dkt == MAXTK && dvt == MAXTV && group > first_plain && group * TG + TG <= n_tiles &&
+               last <= pos_hi && block_of(last) - first_block < cached;
+    };
+    const int lane_k = col * dk + 4 * q4, lane_v = col * bs + 4 * q4;
+    const bool sloped = a.slopes != nullptr;
+    auto scores = [&](auto plain_tag, int uu, int m, int group, float sc[TG][4]) {
+        constexpr bool PLAIN = decltype(plain_tag)::value;
         s16x4 kf[TG][MAXTK];
         const bf16* kbase = a.k_pool + (size_t)(u_kvh[uu] * MAPS + m) * bs * dk + 4 * q4;
+        if constexpr (PLAIN) {
+            const int head = __builtin_amdgcn_readfirstlane(u_kvh[uu]) * MAPS + m;
+#pragma unroll
+            for (int tt = 0; tt < TG; ++tt) {
+                const int j0 = tile_start(group * TG + tt), block = block_of(j0);
+                const int page = __builtin_amdgcn_readfirstlane(pages_s[block - first_block]);
+                const bf16* tile = a.k_pool + (size_t)page * k_page + ((size_t)head * bs + (j0 - block * bs)) * dk;
+#pragma unroll
+                for (int t = 0; t < MAXTK; ++t) kf[tt][t] = load4(tile + lane_k + 16 * t);
+            }
+        } else {
 #pragma unroll
         for (int tt = 0; tt < TG; ++tt) {
             const int j = tile_start(group * TG + tt) + col;  // the key whose row this lane brings
@@ -183,13 +210,12 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
             const int got = page_at(block);
             const int page = j <= pos_hi ? got : -1;
             const bf16* krow = kbase + (size_t)(page < 0 ? 0 : page) * k_page + (jj - block * bs) * dk;
-            // (a group that lies among the reachable keys, with keys as wide as the kernel's tiles, needs no zeros)
-            const bool plain_k = dkt == MAXTK && group > first_plain && tile_start(group * TG + TG - 1) + 15 <= pos_hi;
 #pragma unroll
             for (int t = 0; t < MAXTK; ++t) {
                 const s16x4 k = load4(krow + (t < dkt ? 16 * t : 0));
-                kf[tt][t] = (plain_k || (page >= 0 && t < dkt)) ? k : s16x4{0, 0, 0, 0};
+                kf[tt][t] = (page >= 0 && t < dkt) ? k : s16x4{0, 0, 0, 0};
             }
+        }
         }
         const int pos = u_pos[uu];
 #pragma unroll
@@ -204,7 +230,10 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
             // column of padding then holds numbers that nobody reads
             const bool whole = j0 + 15 <= u_pmin[uu] && (a.chunk <= 0 || j0 >= u_pmax[uu] / a.chunk * a.chunk) &&
                                (a.window <= 0 || u_pmax[uu] - j0 < a.window);
-            if (whole) {
+            if (whole && !sloped) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) sc[tt][r] = acc[r] * scale2;
+            } else if (whole) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) sc[tt][r] = acc[r] * scale2 - u_slope[uu] * (dist0 - (float)r);
             } else {
@@ -219,7 +248,20 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
         }
     };
     // the values of key/value head u_kvh for one group: per tile, keys j0 + 4 q4 .. + 3 of dimension 16 t + col
-    auto load_values = [&](int uu, int group, s16x4 vf[TG][MAXTV]) {
+    auto load_values = [&](auto plain_tag, int uu, int group, s16x4 vf[TG][MAXTV]) {
+        constexpr bool PLAIN = decltype(plain_tag)::value;
+        if constexpr (PLAIN) {
+            const int head = __builtin_amdgcn_readfirstlane(u_kvh[uu]);
+#pragma unroll
+            for (int tt = 0; tt < TG; ++tt) {
+                const int j0 = tile_start(group * TG + tt), block = block_of(j0);
+                const int page = __builtin_amdgcn_readfirstlane(pages_s[block - first_block]);
+                const bf16* tile = a.v_pool + (size_t)page * v_page + (size_t)head * dv * bs + (j0 - block * bs);
+#pragma unroll
+                for (int t = 0; t < MAXTV; ++t) vf[tt][t] = load4(tile + lane_v + (size_t)16 * t * bs);
+            }
+            return;
+        }
         const bf16* vbase = a.v_pool + ((size_t)u_kvh[uu] * dv + col) * bs;
 #pragma unroll
         for (int tt = 0; tt < TG; ++tt) {
@@ -230,20 +272,14 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
             const int page = key < end ? got : -1;
             const int keep = end - key;  // keys behind the request's end hold nothing
             const bf16* vrow = vbase + (size_t)(page < 0 ? 0 : page) * v_page + (kk - block * bs);
-            const bool plain_v = dvt == MAXTV && group > first_plain && tile_start(group * TG + TG - 1) + 15 < end;
-            if (plain_v) {
 #pragma unroll
-                for (int t = 0; t < MAXTV; ++t) vf[tt][t] = load4(vrow + (size_t)16 * t * bs);
-            } else {
-#pragma unroll
-                for (int t = 0; t < MAXTV; ++t) {
-                    const s16x4 got_v = load4(vrow + (t < dvt ? (size_t)16 * t * bs : 0));
-                    s16x4 v = (page >= 0 && t < dvt) ? got_v : s16x4{0, 0, 0, 0};
-                    v.y = keep < 2 ? (short)0 : v.y;
-                    v.z = keep < 3 ? (short)0 : v.z;
-                    v.w = keep < 4 ? (short)0 : v.w;
-                    vf[tt][t] = v;
-                }
+            for (int t = 0; t < MAXTV; ++t) {
+                const s16x4 got_v = load4(vrow + (t < dvt ? (size_t)16 * t * bs : 0));
+                s16x4 v = (page >= 0 && t < dvt) ? got_v : s16x4{0, 0, 0, 0};
+                v.y = keep < 2 ? (short)0 : v.y;
+                v.z = keep < 3 ? (short)0 : v.z;
+                v.w = keep < 4 ? (short)0 : v.w;
+                vf[tt][t] = v;
             }
         }
     };
@@ -291,24 +327,30 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
         for (int round = 0; round < n_rounds; ++round) {
             const int group = (round * NS + slice) * NSG + share;
             if (group >= n_groups) break;  // (nothing left for this slice)
+            auto walk = [&](auto plain_tag) {
 #pragma unroll
-            for (int uu = 0; uu < MAXU; ++uu) {
-                if (!mine[uu]) continue;
-                s16x4 vf[TG][MAXTV];
+                for (int uu = 0; uu < MAXU; ++uu) {
+                    if (!mine[uu]) continue;
+                    s16x4 vf[TG][MAXTV];
 #pragma unroll
-                for (int m = 0; m < MAPS; ++m) {
-                    float sc[TG][4], p[TG][4];
-                    if (m == 0) load_values(uu, group, vf);  // (asked for beside the keys; both maps use them)
-                    scores(uu, m, group, sc);
-                    const float corr = join(sc, run_m[uu][m], run_l[uu][m], p);
-                    s16x4 pf[TG];
+                    for (int m = 0; m < MAPS; ++m) {
+                        float sc[TG][4], p[TG][4];
+                        if (m == 0) load_values(plain_tag, uu, group, vf);  // (asked for beside the keys; both maps use them)
+                        scores(plain_tag, uu, m, group, sc);
+                        const float corr = join(sc, run_m[uu][m], run_l[uu][m], p);
+                        s16x4 pf[TG];
 #pragma unroll
-                    for (int tt = 0; tt < TG; ++tt) pf[tt] = pack4(p[tt][0], p[tt][1], p[tt][2], p[tt][3]);
+                        for (int tt = 0; tt < TG; ++tt) pf[tt] = pack4(p[tt][0], p[tt][1], p[tt][2], p[tt][3]);
+                        if (__any(corr != 1.f)) {  // (no column's maximum moved: nothing to scale)
 #pragma unroll
-                    for (int t = 0; t < MAXTV; ++t) acc_o[uu][m][t] *= corr;
-                    times_values(vf, pf, acc_o[uu][m]);
+                            for (int t = 0; t < MAXTV; ++t) acc_o[uu][m][t] *= corr;
+                        }
+                        times_values(vf, pf, acc_o[uu][m]);
+                    }
                 }
-            }
+            };
+            if (plain_group(group)) walk(std::true_type{});
+            else walk(std::false_type{});
         }
 #pragma unroll
         for (int uu = 0; uu < MAXU; ++uu)
@@ -365,13 +407,16 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
         for (int round = 0; round < (a.mode == 2 ? 0 : n_rounds); ++round) {
             const int group = (round * NS + slice) * NSG + share;
             if (group >= n_groups) break;  // (nothing left for this slice)
+            auto walk = [&](auto plain_tag) {
 #pragma unroll
-            for (int uu = 0; uu < MAXU; ++uu) {
-                if (!mine[uu]) continue;
-                float sc[TG][4], p[TG][4];
-                scores(uu, 0, group, sc);
-                join(sc, run_m[uu][0], run_l[uu][0], p);
-            }
+                for (int uu = 0; uu < MAXU; ++uu) {
+                    if (!mine[uu]) continue;
+                    float sc[TG][4], p[TG][4];
+                    scores(plain_tag, uu, 0, group, sc);
+                    join(sc, run_m[uu][0], run_l[uu][0], p);
+                }
+            };
+            walk(std::false_type{});
         }
         float inv_l[MAXU];
 #pragma unroll
@@ -423,21 +468,24 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
             const int group = (round * NS + slice) * NSG + share;
             const bool some = group < n_groups;  // (a slice without keys at this turn of the loop only keeps the barriers' count)
             s16x4 vf[MAXU][TG][MAXTV];
+            auto walk = [&](auto plain_tag) {
 #pragma unroll
-            for (int uu = 0; uu < MAXU; ++uu) {
-                if (!mine[uu] || !some) continue;
-                float sc[TG][4];
-                load_values(uu, group, vf[uu]);
-                scores(uu, 0, group, sc);
+                for (int uu = 0; uu < MAXU; ++uu) {
+                    if (!mine[uu]) continue;
+                    float sc[TG][4];
+                    load_values(plain_tag, uu, group, vf[uu]);
+                    scores(plain_tag, uu, 0, group, sc);
 #pragma unroll
-                for (int tt = 0; tt < TG; ++tt) {
-                    f32x4 w;
+                    for (int tt = 0; tt < TG; ++tt) {
+                        f32x4 w;
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) w[r] = fast_exp2(sc[tt][r] - run_m[uu][0]) * inv_l[uu];
-                    if (col < used_cols)
-                        *reinterpret_cast<f32x4*>(pbuf + ((size_t)u_tl[uu] * H + u_h[uu]) * group_keys + 16 * tt + 4 * q4) = w;
+                        for (int r = 0; r < 4; ++r) w[r] = fast_exp2(sc[tt][r] - run_m[uu][0]) * inv_l[uu];
+                        if (col < used_cols)
+                            *reinterpret_cast<f32x4*>(pbuf + ((size_t)u_tl[uu] * H + u_h[uu]) * group_keys + 16 * tt + 4 * q4) = w;
+                    }
                 }
-            }
+            };
+            if (some) walk(std::false_type{});
             __syncthreads();
 #pragma unroll
             for (int uu = 0; uu < MAXU; ++uu) {
@@ -527,18 +575,19 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
     }
 }
 
-// out[row] = the sum of the shares' parts, rounded once; one workgroup per request of one token
+// out[row] = the sum of the shares' parts, rounded once; the workgroups (request, y) take the request's rows in turn
 __global__ __launch_bounds__(256) void add_shares_kernel(bf16* __restrict__ out, int out_stride, const float* __restrict__ ws_o,
                                                          int ws_rows, int shares, int width, const int* __restrict__ cu_seqlens,
                                                          const int* __restrict__ context_lens, int seq_begin) {
     const int b = seq_begin + blockIdx.x;
     if (context_lens[b] <= 0) return;
-    const int row = cu_seqlens[b];
-    for (int c = 4 * threadIdx.x; c < width; c += 4 * 256) {
-        f32x4 sum = {0.f, 0.f, 0.f, 0.f};
-        for (int s2 = 0; s2 < shares; ++s2) sum += *reinterpret_cast<const f32x4*>(ws_o + ((size_t)s2 * ws_rows + row) * width + c);
-        *reinterpret_cast<s16x4*>(out + (size_t)row * out_stride + c) = pack4(sum[0], sum[1], sum[2], sum[3]);
-    }
+    for (int row = cu_seqlens[b] + blockIdx.y; row < cu_seqlens[b + 1]; row += gridDim.y)
+        for (int c = 4 * threadIdx.x; c < width; c += 4 * 256) {
+            f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+            for (int s2 = 0; s2 < shares; ++s2)
+                sum += *reinterpret_cast<const f32x4*>(ws_o + ((size_t)s2 * ws_rows + row) * width + c);
+            *reinterpret_cast<s16x4*>(out + (size_t)row * out_stride + c) = pack4(sum[0], sum[1], sum[2], sum[3]);
+        }
 }
 
 // tiles in a group: 4 (64 keys) up to sizes of 64; wider keys or values leave registers for 2
@@ -564,6 +613,17 @@ static int launch(const MfmaArgs& a, dim3 grid, int threads, size_t lds, hipStre
 
 extern "C" {
 
+// Tokens one workgroup takes when heads are mixed (what a caller needs to count the workgroups of a launch).
+int llms_attend_composed_mfma_tokens(int heads, int kv_heads, int dk, int dv, int max_new) {
+    if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || heads / kv_heads > 16 || kv_heads > 32) return 0;
+    const int tpw = 16 / (heads / kv_heads);
+    const int group_keys = 16 * ((dk > 64 || dv > 64) ? 2 : 4);
+    int upk = 32 / kv_heads;
+    while (upk > 1 && (size_t)upk * tpw * heads * group_keys * sizeof(float) > 64 * 1024) --upk;
+    while (upk > 1 && (upk - 1) * tpw >= max_new) --upk;
+    return upk * tpw;
+}
+
 // Rows [token rows of requests seq_begin .. seq_begin + n_seqs) of q and out; `max_new`: most tokens one of them brings.
 int llms_attend_composed_mfma(void* out, int out_stride, const void* q, int q_stride, const void* k_pool,
                               const void* v_pool, const int* block_tables, const int* table_rows, int max_blocks,
@@ -585,7 +645,7 @@ int llms_attend_composed_mfma(void* out, int out_stride, const void* q, int q_st
     a.out = (bf16*)out, a.q = (const bf16*)q, a.k_pool = (const bf16*)k_pool, a.v_pool = (const bf16*)v_pool;
     a.block_tables = block_tables, a.table_rows = table_rows, a.cu_seqlens = cu_seqlens, a.context_lens = context_lens;
     a.slopes = slopes, a.talk = talk;
-    a.out_stride = out_stride, a.q_stride = q_stride, a.max_blocks = max_blocks, a.seq_begin = seq_begin;
+    a.out_stride = out_stride, a.q_stride = q_stride, a.max_blocks = max_blocks, a.seq_begin = seq_begin, a.n_seqs = n_seqs;
     a.heads = heads, a.kv_heads = kv_heads, a.grp = heads / kv_heads, a.dk = dk, a.dv = dv, a.block_size = block_size;
     a.window = window, a.keep_first = keep_first, a.chunk = chunk;
     a.scale = scale, a.lambda = lambda, a.eps = eps, a.out_scale = out_scale, a.head_norm = head_norm;
@@ -613,7 +673,7 @@ int llms_attend_composed_mfma(void* out, int out_stride, const void* q, int q_st
         const size_t lds = (floats + AM_PAGE_CACHE) * sizeof(float);
         LLMS_REQUIRE(lds <= 160 * 1024, "attend_composed_mfma: too many heads for the LDS");
         dim3 grid(n_seqs * a.blocks_per_seq, 1);
-        if (shares > 1 && upk == 1 && max_new == 1) {  // single tokens: every request's keys go to `shares` workgroups
+        if (shares > 1) {  // the keys of every block of tokens go to `shares` workgroups
             LLMS_REQUIRE(ws_stats && ws_o && ws_rows > 0 && shares <= 64, "attend_composed_mfma: shares need their workspaces");
             a.shares = shares;
             grid.z = shares;
@@ -622,8 +682,8 @@ int llms_attend_composed_mfma(void* out, int out_stride, const void* q, int q_st
                                             : launch<1, true, 1, 1024>(a, grid, waves * LLMS_WAVE, lds, stream);
                 if (rc != LLMS_OK) return rc;
             }
-            add_shares_kernel<<<n_seqs, 256, 0, stream>>>(a.out, out_stride, ws_o, ws_rows, shares, heads * dv, cu_seqlens,
-                                                          context_lens, seq_begin);
+            add_shares_kernel<<<dim3(n_seqs, max_new < 64 ? max_new : 64), 256, 0, stream>>>(
+                a.out, out_stride, ws_o, ws_rows, shares, heads * dv, cu_seqlens, context_lens, seq_begin);
             LLMS_LAUNCH_CHECK();
         }
         if (a.units > 16) return launch<1, true, 2, 1024>(a, grid, waves * LLMS_WAVE, lds, stream);

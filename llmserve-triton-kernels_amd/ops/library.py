@@ -972,6 +972,12 @@ def attend_composed_mfma_supported(dtype: torch.dtype, heads: int, kv_heads: int
     return True
 
 
+def attend_composed_mfma_tokens(heads: int, kv_heads: int, dk: int, dv: int, max_new: int) -> int:
+    """Tokens one workgroup of `attend_composed_mfma` takes when heads are mixed (0: sizes it does not take)."""
+    return int(load("attention_composed_mfma").llms_attend_composed_mfma_tokens(
+        c_int(heads), c_int(kv_heads), c_int(dk), c_int(dv), c_int(max_new)))
+
+
 def attend_composed_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                          block_tables: torch.Tensor, cu_seqlens: torch.Tensor, context_lens: torch.Tensor,
                          seq_begin: int, n_seqs: int, max_new: int, *, heads: int, kv_heads: int, dk: int, dv: int,
@@ -982,9 +988,9 @@ def attend_composed_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tenso
     """`attend_composed` on the matrix cores (bfloat16) for requests [seq_begin, seq_begin + n_seqs) of a step: request
     b owns rows cu_seqlens[b] .. cu_seqlens[b+1] of q and out, brings at most `max_new` tokens and is context_lens[b]
     long after the step (0: padding, left alone).  Same arguments and arithmetic otherwise; the weights are rounded
-    to bfloat16 as the operand of the value product.  `shares` > 1 (requests of one token whose heads' weights are
-    mixed): every request's keys are shared out to that many workgroups in two launches (maxima and sums; weights
-    and values), their 32-bit parts added up by a third."""
+    to bfloat16 as the operand of the value product.  `shares` > 1 (where the heads' weights are mixed): the keys
+    of every block of tokens are shared out to that many workgroups in two launches (maxima and sums; weights and
+    values), their 32-bit parts added up by a third."""
     dev = _dev(out, q, k_pool, v_pool, block_tables, cu_seqlens, context_lens, slopes, talk, table_rows)
     if not attend_composed_mfma_supported(q.dtype, heads, kv_heads, dk, dv, block_size, talk is not None):
         raise ValueError("attend_composed_mfma does not take these sizes; see attend_composed_mfma_supported")
@@ -1020,7 +1026,7 @@ def attend_composed_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tenso
     if n_seqs == 0 or max_new <= 0 or q.shape[0] == 0:
         return out
     ws_stats = ws_o = None
-    if not (shares > 1 and talk is not None and max_new == 1):
+    if not (shares > 1 and talk is not None):
         shares = 1
     else:
         shares = min(int(shares), 64)

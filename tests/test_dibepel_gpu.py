@@ -290,7 +290,7 @@ def attend_mfma(seqs, bs, shares=1, **kw):
     if n_dec:
         ops.attend_composed_mfma(*args, 0, n_dec, 1, shares=shares, **common)
     if n_dec < len(seqs):
-        ops.attend_composed_mfma(*args, n_dec, len(seqs) - n_dec, max(n for *_x, n in seqs), **common)
+        ops.attend_composed_mfma(*args, n_dec, len(seqs) - n_dec, max(n for *_x, n in seqs), shares=shares, **common)
     return [out[cu[i]: cu[i + 1]] for i in range(len(seqs))]
 
 
@@ -348,11 +348,11 @@ def test_matrix_core_kernel_mixed_heads(heads, kv, dk, dv, chunk, bs):
                       talk=talk.float().to(DEV))
     for i, (g, r) in enumerate(zip(got, refs)):
         close(g, r, dt, f"request {i}")
-    # the keys of the requests of one token shared out to several workgroups
+    # every request's keys shared out to several workgroups: single tokens and portions of prompts alike
     for shares in (2, 5):
-        got = attend_mfma(seqs[:2], bs, shares=shares, heads=heads, kv_heads=kv, chunk=chunk or 0, scale=0.3,
+        got = attend_mfma(seqs, bs, shares=shares, heads=heads, kv_heads=kv, chunk=chunk or 0, scale=0.3,
                           slopes=slopes.float().to(DEV), talk=talk.float().to(DEV))
-        for i, (g, r) in enumerate(zip(got, refs[:2])):
+        for i, (g, r) in enumerate(zip(got, refs)):
             close(g, r, dt, f"request {i} in {shares} shares")
     got = attend_mfma(seqs[2:3], bs, heads=heads, kv_heads=kv, chunk=chunk or 0, scale=0.3)  # neither slopes nor mixing
     ref = pd.talking_heads(seqs[2][0].double(), seqs[2][1].double(), seqs[2][2].double(), pd.visible_chunk(90, chunk), 0.3,
