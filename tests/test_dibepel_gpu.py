@@ -495,3 +495,60 @@ def test_named_sizes_run_from_the_command_line_entry(capsys):
 
     assert main(["--model", "dibepel-tiny", "--random-weights", "--max-new-tokens", "5", "--dtype", "float32"]) == 0
     assert "decode=" in capsys.readouterr().out
+
+
+def drawn_config(seed: int) -> tuple[dict, int]:
+    """A configuration drawn at random from what config.json allows: layer kinds in any order, some layers on
+    another's tensors, some without feed-forward, 1 to 16 query heads per key/value head, key and value sizes that
+    the matrix-core kernel takes (multiples of 16) and that it does not, windows, kept tokens and chunks from 1 key
+    up, 1 to 5 taps; and a page size."""
+    import random
+
+    rng = random.Random(seed)
+    sizes = [8, 16, 16, 24, 32, 40, 48, 64]
+    layers = []
+    for i in range(rng.randint(2, 5)):
+        kind = rng.choice(["attention", "attention_2"])
+        kv = rng.choice([1, 1, 2, 3, 4])
+        heads = kv * rng.choice([1, 1, 2, 4, 8, 16] if kv == 1 else [1, 2, 3])
+        mixer = {"heads": heads, "kv_heads": kv, "dim": rng.choice(sizes), "vdim": rng.choice(sizes),
+                 "scale": rng.choice([0.1, 0.2, 0.35])}
+        if kind == "attention":
+            mixer["diff"] = rng.choice([0.0, 0.2, 0.5, 0.8])
+            mixer["mask"] = {} if rng.random() < 0.15 else {"size": rng.choice([1, 2, 7, 16, 33, 64]),
+                                                            "keep_first": rng.choice([0, 1, 5, 16, 40])}
+        else:
+            mixer["conv"] = rng.randint(1, 5)
+            mixer["mask"] = {} if rng.random() < 0.15 else {"size": rng.choice([1, 3, 16, 31, 64, 100])}
+        changes = {"mixer": mixer}
+        if rng.random() < 0.25:
+            changes["mlp"] = None
+        layers.append((kind, changes))
+    for _ in range(rng.randint(0, 3)):  # further runs of earlier layers, appended (so no index moves)
+        src = rng.randrange(len(layers))
+        layers.append((layers[src][0], {"weights_of": src}))  # (a layer that itself runs on another's tensors makes a chain)
+    width = rng.choice([40, 64, 72, 100])
+    return config_of(width=width, vocab=rng.choice([61, 128, 257]), scale=rng.choice([0.5, 1.0, 2.5]),
+                     eps=rng.choice([1e-6, 1e-5]), ff=rng.choice([24, 64, 120]), layers=layers), rng.choice([4, 8, 16])
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_configurations_drawn_at_random(tmp_path, seed):
+    from llmserve.config import EngineConfig
+    from llmserve.engine.runner import ModelRunner
+
+    config, bs = drawn_config(seed)
+    w = write_model(tmp_path, config, seed=900 + seed)
+    seqs = {f"q{i}": traces.random_ids(config["vocab"], n, 40 * seed + i) for i, n in enumerate([90, 3, 47, 130, 18])}
+    ref = {rid: pd.forward(config, w, ids) for rid, ids in seqs.items()}
+    for dtype_name in ("float32", "bfloat16"):
+        steps = traces.mixed(seqs, seed=seed, live_max=3, tail=30)
+        pages = -(-traces.tokens_needed(steps, round_to=bs) // bs)
+        runner = ModelRunner.from_folder(tmp_path, EngineConfig(dtype=dtype_name, block_size=bs, num_blocks=pages,
+                                                                max_num_seqs=3))
+        runner.storage.poison()
+        got = run_trace(runner, steps)
+        for rid in seqs:
+            logits_close(got[rid], ref[rid], getattr(torch, dtype_name), f"seed {seed} {rid} {dtype_name}: {config['layers']}")
+        assert runner.manager.num_free_slots == 3
+        assert all(a.num_free == pages for a in runner.manager.allocators.values())
