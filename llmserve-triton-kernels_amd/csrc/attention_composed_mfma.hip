@@ -662,8 +662,8 @@ int llms_attend_composed_mfma(void* out, int out_stride, const void* q, int q_st
         while (upk > 1 && (upk - 1) * a.tpw >= max_new) --upk;  // (no more tokens than the longest portion has)
         a.upk = upk, a.tok = upk * a.tpw, a.kv_per_wg = kv_heads, a.units = kv_heads * upk;
         a.slices = 1;
-        if (upk == 1)  // few tokens (decoding): the groups of keys are dealt to several waves per unit
-            while (a.slices < 4 && a.units * a.slices * 2 <= 16) a.slices *= 2;
+        if (upk == 1 && shares <= 1)  // few tokens (decoding) in one workgroup: the groups of keys are dealt to several waves
+            while (a.slices < 4 && a.units * a.slices * 2 <= 16) a.slices *= 2;  // per unit (with shares: to workgroups)
         const int unit_waves = a.units > 16 ? (a.units + 1) / 2 : a.units;
         const int waves = unit_waves * a.slices;
         a.blocks_per_seq = (max_new + a.tok - 1) / a.tok;
