@@ -366,8 +366,9 @@ def write_model(folder, config, seed):
 
     from llmserve.weights import write_random_model
 
-    # weights large enough for attention to have favourites and for gates to leave one half
-    write_random_model(folder, config, seed=seed, std=0.08, norm_std=0.02)
+    # weights large enough for attention to have favourites and for gates to leave one half; stored in bfloat16, so
+    # that both engines and the plain implementation hold the same numbers and only the arithmetic differs
+    write_random_model(folder, config, seed=seed, dtype=torch.bfloat16, std=0.08, norm_std=0.02)
     return {k: v.double() for k, v in load_file(str(folder / "model.safetensors")).items()}
 
 
