@@ -300,6 +300,9 @@ MFMA_DIFF = [  # heads, kv_heads, dk, dv, window, keep_first, block size
     (16, 2, 64, 128, 33, 0, 16),
     (3, 1, 16, 16, None, 0, 4),  # three heads in a unit of 16 columns: five tokens and a padded column
     (16, 1, 16, 32, 21, 3, 8),  # sixteen heads on one key/value head: a unit is one token
+    (2, 1, 128, 128, 50, 9, 16),  # the widest keys and values the kernel takes
+    (4, 4, 128, 64, 1000, 0, 16),
+    (8, 2, 96, 112, 37, 20, 8),
 ]
 
 
@@ -329,6 +332,9 @@ MFMA_TALK = [  # heads, kv_heads, dk, dv, chunk, block size
     (6, 2, 16, 16, 50, 4),
     (16, 1, 32, 16, 40, 8),  # a unit is one token
     (24, 24, 16, 16, 30, 16),  # 24 units in 12 waves
+    (4, 2, 128, 128, 70, 16),  # the widest keys and values the kernel takes
+    (20, 20, 128, 128, 64, 16),  # ... with two units a wave
+    (8, 4, 80, 96, 33, 8),
 ]
 
 
