@@ -4,7 +4,9 @@
 //                 causal convolution per channel (from 2 taps on the request's last taps - 1 projected rows lie in its
 //                 state, a ring indexed by position), is rounded once, and lands in the query rows and at the tokens'
 //                 cache slots.  taps = 1: a factor per channel; taps = 0: rounding and store alone.
-//   conv_state    the ring takes the last taps - 1 projected rows of every request of the step.
+//   conv_state    the ring takes the last taps - 1 projected rows of every request of the step (a kernel of its own,
+//                 because a token's write would race with its neighbours' reads; when every request brings one
+//                 token, conv_store writes the ring itself).
 //   attend        one workgroup per new token, all heads.  Score heads s = h * maps + m (maps = 2: two score maps
 //                 per query head over the same values); s reads key head (h / (H / G)) * maps + m, values come from
 //                 value head h / (H / G).  A query at position i sees the key j <= i if
@@ -29,7 +31,7 @@ __global__ __launch_bounds__(AC_THREADS) void conv_store_kernel(
     int taps, const float* __restrict__ state, size_t state_slot_stride, const int* __restrict__ state_slots,
     const int* __restrict__ token_seq, const int* __restrict__ positions, const int* __restrict__ cu_seqlens,
     const int* __restrict__ slots, T* __restrict__ k_pool, T* __restrict__ v_pool, int cq, int ck, int cv, int k_heads,
-    int dk, int v_heads, int dv, int block_size) {
+    int dk, int v_heads, int dv, int block_size, float* __restrict__ state_out, const int* __restrict__ context_lens) {
     const int n = blockIdx.x;
     const int c = blockIdx.y * AC_THREADS + threadIdx.x;
     const int channels = cq + ck + cv;
@@ -51,6 +53,11 @@ __global__ __launch_bounds__(AC_THREADS) void conv_store_kernel(
                 u = ring[(size_t)(pos % (taps - 1)) * channels + c];
             y = fmaf(taps_w[(size_t)c * taps + j], u, y);
         }
+        // every request brings one token: the ring takes the token's own row here (nobody else reads this request's
+        // ring in this launch, and this thread has read the place it overwrites); a request of length 0 is padding
+        if (state_out && taps > 1 && context_lens[b] > 0)
+            state_out[(size_t)state_slots[b] * state_slot_stride + (size_t)(p % (taps - 1)) * channels + c] =
+                proj[(size_t)n * proj_stride + c];
     } else {
         y = proj[(size_t)n * proj_stride + c];
     }
@@ -280,22 +287,26 @@ extern "C" {
 int llms_conv_store(int dtype, void* q_out, int q_stride, const float* proj, int proj_stride, const float* taps_w, int taps,
                     const float* state, size_t state_slot_stride, const int* state_slots, const int* token_seq,
                     const int* positions, const int* cu_seqlens, const int* slots, void* k_pool, void* v_pool, int n_tokens,
-                    int cq, int ck, int cv, int k_heads, int dk, int v_heads, int dv, int block_size, hipStream_t stream) {
+                    int cq, int ck, int cv, int k_heads, int dk, int v_heads, int dv, int block_size, float* state_out,
+                    const int* context_lens, hipStream_t stream) {
     LLMS_REQUIRE(n_tokens > 0 && cq > 0 && ck >= 0 && cv >= 0, "conv_store: sizes must be positive");
     LLMS_REQUIRE(ck == k_heads * dk && cv == v_heads * dv, "conv_store: channels do not match heads times sizes");
     LLMS_REQUIRE(taps < 1 || (taps_w && token_seq && positions && cu_seqlens),
                  "conv_store: a convolution needs its taps and the batch's arrays");
     LLMS_REQUIRE(taps <= 1 || (state && state_slots), "conv_store: a convolution of two taps or more needs the state");
     LLMS_REQUIRE(!slots || (k_pool && v_pool && block_size > 0), "conv_store: slots given without pools");
+    LLMS_REQUIRE(!state_out || (context_lens && state_out == state), "conv_store: the ring is updated in place, with the requests' lengths at hand");
     dim3 grid(n_tokens, (cq + ck + cv + AC_THREADS - 1) / AC_THREADS);
     if (dtype == 0)
         conv_store_kernel<float><<<grid, AC_THREADS, 0, stream>>>(
             (float*)q_out, q_stride, proj, proj_stride, taps_w, taps, state, state_slot_stride, state_slots, token_seq,
-            positions, cu_seqlens, slots, (float*)k_pool, (float*)v_pool, cq, ck, cv, k_heads, dk, v_heads, dv, block_size);
+            positions, cu_seqlens, slots, (float*)k_pool, (float*)v_pool, cq, ck, cv, k_heads, dk, v_heads, dv, block_size,
+            state_out, context_lens);
     else if (dtype == 1)
         conv_store_kernel<bf16><<<grid, AC_THREADS, 0, stream>>>(
             (bf16*)q_out, q_stride, proj, proj_stride, taps_w, taps, state, state_slot_stride, state_slots, token_seq,
-            positions, cu_seqlens, slots, (bf16*)k_pool, (bf16*)v_pool, cq, ck, cv, k_heads, dk, v_heads, dv, block_size);
+            positions, cu_seqlens, slots, (bf16*)k_pool, (bf16*)v_pool, cq, ck, cv, k_heads, dk, v_heads, dv, block_size,
+            state_out, context_lens);
     else
         LLMS_REQUIRE(false, "conv_store: dtype must be 0 (float32) or 1 (bfloat16)");
     LLMS_LAUNCH_CHECK();

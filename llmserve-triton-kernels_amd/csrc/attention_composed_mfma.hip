@@ -575,19 +575,25 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
     }
 }
 
-// out[row] = the sum of the shares' parts, rounded once; the workgroups (request, y) take the request's rows in turn
+// out[row] = the sum of the shares' parts (up to 16), rounded once.  The workgroups (request, y, z) take the request's
+// rows in turn (y) and 1,024 columns each (z); a thread asks for all shares of its 4 columns before it adds them up.
 __global__ __launch_bounds__(256) void add_shares_kernel(bf16* __restrict__ out, int out_stride, const float* __restrict__ ws_o,
                                                          int ws_rows, int shares, int width, const int* __restrict__ cu_seqlens,
                                                          const int* __restrict__ context_lens, int seq_begin) {
     const int b = seq_begin + blockIdx.x;
     if (context_lens[b] <= 0) return;
-    for (int row = cu_seqlens[b] + blockIdx.y; row < cu_seqlens[b + 1]; row += gridDim.y)
-        for (int c = 4 * threadIdx.x; c < width; c += 4 * 256) {
-            f32x4 sum = {0.f, 0.f, 0.f, 0.f};
-            for (int s2 = 0; s2 < shares; ++s2)
-                sum += *reinterpret_cast<const f32x4*>(ws_o + ((size_t)s2 * ws_rows + row) * width + c);
-            *reinterpret_cast<s16x4*>(out + (size_t)row * out_stride + c) = pack4(sum[0], sum[1], sum[2], sum[3]);
-        }
+    const int c = 4 * (blockIdx.z * 256 + threadIdx.x);
+    if (c >= width) return;
+    for (int row = cu_seqlens[b] + blockIdx.y; row < cu_seqlens[b + 1]; row += gridDim.y) {
+        f32x4 part[16];
+#pragma unroll
+        for (int s2 = 0; s2 < 16; ++s2)  // (a share that does not exist reads the last one and counts for nothing)
+            part[s2] = *reinterpret_cast<const f32x4*>(ws_o + ((size_t)(s2 < shares ? s2 : shares - 1) * ws_rows + row) * width + c);
+        f32x4 sum = part[0];
+#pragma unroll
+        for (int s2 = 1; s2 < 16; ++s2) sum += s2 < shares ? part[s2] : f32x4{0.f, 0.f, 0.f, 0.f};
+        *reinterpret_cast<s16x4*>(out + (size_t)row * out_stride + c) = pack4(sum[0], sum[1], sum[2], sum[3]);
+    }
 }
 
 // tiles in a group: 4 (64 keys) up to sizes of 64; wider keys or values leave registers for 2
@@ -674,7 +680,7 @@ int llms_attend_composed_mfma(void* out, int out_stride, const void* q, int q_st
         LLMS_REQUIRE(lds <= 160 * 1024, "attend_composed_mfma: too many heads for the LDS");
         dim3 grid(n_seqs * a.blocks_per_seq, 1);
         if (shares > 1) {  // the keys of every block of tokens go to `shares` workgroups
-            LLMS_REQUIRE(ws_stats && ws_o && ws_rows > 0 && shares <= 64, "attend_composed_mfma: shares need their workspaces");
+            LLMS_REQUIRE(ws_stats && ws_o && ws_rows > 0, "attend_composed_mfma: shares need their workspaces");
             a.shares = shares;
             grid.z = shares;
             for (a.mode = 1; a.mode <= 2; ++a.mode) {
@@ -682,7 +688,8 @@ int llms_attend_composed_mfma(void* out, int out_stride, const void* q, int q_st
                                             : launch<1, true, 1, 1024>(a, grid, waves * LLMS_WAVE, lds, stream);
                 if (rc != LLMS_OK) return rc;
             }
-            add_shares_kernel<<<dim3(n_seqs, max_new < 64 ? max_new : 64), 256, 0, stream>>>(
+            LLMS_REQUIRE(shares <= 16, "attend_composed_mfma: up to 16 shares");
+            add_shares_kernel<<<dim3(n_seqs, max_new < 64 ? max_new : 64, (heads * dv + 1023) / 1024), 256, 0, stream>>>(
                 a.out, out_stride, ws_o, ws_rows, shares, heads * dv, cu_seqlens, context_lens, seq_begin);
             LLMS_LAUNCH_CHECK();
         }

@@ -3,6 +3,7 @@
 //   rmsnorm32        y[r] = x[s] * rsqrt(mean(x[s]^2) + eps) * (offset + w), s = rows[r] or r   (x float, y T)
 //   gated_add        x[n] += sum over branches b of g_b * y_b[n]                    (all float)
 //                    g_b = sigmoid(z_b[n] + bias_b) where the branch has a gate, else 1
+//   gated_add_norm   the same sum and, in the same kernel, the norm of the summed row for the next layer
 // T is float or bfloat16.  One workgroup per row; every reduction has an order fixed by the sizes alone.
 #include "common.h"
 
@@ -90,6 +91,60 @@ __global__ __launch_bounds__(S32_THREADS) void gated_add_vec_kernel(float* __res
     r.z = xv.z + (g0.z * a0.z + g1.z * a1.z);
     r.w = xv.w + (g0.w * a0.w + g1.w * a1.w);
     *reinterpret_cast<float4*>(x + (size_t)n * hidden + c) = r;
+}
+
+// gated_add and the norm of the summed row in one kernel (what the next layer reads): x[n] is summed and stored as in
+// gated_add_vec, out[n] = x[n] * rsqrt(mean(x[n]^2) + eps) * (offset + w).  One workgroup a row of up to
+// 4 * S32_VEC * S32_THREADS.
+template <typename T>
+__global__ __launch_bounds__(S32_THREADS) void gated_add_norm_vec_kernel(
+    T* __restrict__ out, float* __restrict__ x, const float* __restrict__ z, int z_stride, int z_col0, int z_col1,
+    const float* __restrict__ bias0, const float* __restrict__ bias1, const float* __restrict__ y0, int y0_stride,
+    const float* __restrict__ y1, int y1_stride, const float* __restrict__ weight, int hidden, float eps, float offset) {
+    __shared__ float lds[16];
+    const int n = blockIdx.x, n4 = hidden / 4;
+    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f), one = make_float4(1.f, 1.f, 1.f, 1.f);
+    auto at = [](const float* p) { return *reinterpret_cast<const float4*>(p); };
+    float4 r[S32_VEC];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < S32_VEC; ++i) {
+        const int c = 4 * (threadIdx.x + i * S32_THREADS);
+        r[i] = zero;
+        if (c < hidden) {
+            const float4 xv = at(x + (size_t)n * hidden + c);
+            const float4 a0 = y0 ? at(y0 + (size_t)n * y0_stride + c) : zero;
+            const float4 a1 = y1 ? at(y1 + (size_t)n * y1_stride + c) : zero;
+            const float4 z0 = (y0 && z_col0 >= 0) ? at(z + (size_t)n * z_stride + z_col0 + c) : zero;
+            const float4 z1 = (y1 && z_col1 >= 0) ? at(z + (size_t)n * z_stride + z_col1 + c) : zero;
+            const float4 b0 = (y0 && z_col0 >= 0 && bias0) ? at(bias0 + c) : zero;
+            const float4 b1 = (y1 && z_col1 >= 0 && bias1) ? at(bias1 + c) : zero;
+            const float4 g0 = (y0 && z_col0 >= 0) ? gate4(z0, b0) : one;
+            const float4 g1 = (y1 && z_col1 >= 0) ? gate4(z1, b1) : one;
+            float4 s;
+            s.x = xv.x + (g0.x * a0.x + g1.x * a1.x);
+            s.y = xv.y + (g0.y * a0.y + g1.y * a1.y);
+            s.z = xv.z + (g0.z * a0.z + g1.z * a1.z);
+            s.w = xv.w + (g0.w * a0.w + g1.w * a1.w);
+            *reinterpret_cast<float4*>(x + (size_t)n * hidden + c) = s;
+            r[i] = s;
+            ss += s.x * s.x + s.y * s.y + s.z * s.z + s.w * s.w;
+        }
+    }
+    const float inv = 1.0f / sqrtf(block_sum(ss, lds) / (float)hidden + eps);
+    T* orow = out + (size_t)n * hidden;
+#pragma unroll
+    for (int i = 0; i < S32_VEC; ++i) {
+        const int c = 4 * (threadIdx.x + i * S32_THREADS);
+        if (c < hidden) {
+            const float4 w = at(weight + c);
+            orow[c + 0] = from_f32<T>(r[i].x * inv * (offset + w.x));
+            orow[c + 1] = from_f32<T>(r[i].y * inv * (offset + w.y));
+            orow[c + 2] = from_f32<T>(r[i].z * inv * (offset + w.z));
+            orow[c + 3] = from_f32<T>(r[i].w * inv * (offset + w.w));
+        }
+    }
+    (void)n4;
 }
 
 template <typename T>
@@ -187,6 +242,29 @@ int llms_gated_add(float* x, const float* z, int z_stride, int z_col0, int z_col
         gated_add_kernel<<<n, S32_THREADS, 0, stream>>>(x, z, z_stride, z_col0, z_col1, bias0, bias1, y0, y0_stride, y1,
                                                         y1_stride, hidden);
     }
+    LLMS_LAUNCH_CHECK();
+}
+
+// 0: launched; 3: the sizes are not what the fused kernel takes (the caller runs gated_add and rmsnorm32 instead)
+int llms_gated_add_norm(int dtype, void* out, float* x, const float* z, int z_stride, int z_col0, int z_col1,
+                        const float* bias0, const float* bias1, const float* y0, int y0_stride, const float* y1,
+                        int y1_stride, const float* weight, float eps, float offset, int n, int hidden, hipStream_t stream) {
+    LLMS_REQUIRE(n > 0 && hidden > 0, "gated_add_norm: sizes must be positive");
+    LLMS_REQUIRE(y0 || y1, "gated_add_norm: no branch to add");
+    LLMS_REQUIRE(z || (z_col0 < 0 && z_col1 < 0), "gated_add_norm: gate columns named without gate products");
+    LLMS_REQUIRE(dtype == 0 || dtype == 1, "gated_add_norm: dtype must be 0 (float32) or 1 (bfloat16)");
+    auto aligned = [](const void* p) { return ((uintptr_t)p % 16) == 0; };
+    const bool vec = hidden % 4 == 0 && hidden <= 4 * S32_VEC * S32_THREADS && z_stride % 4 == 0 && y0_stride % 4 == 0 &&
+                     y1_stride % 4 == 0 && (z_col0 < 0 || z_col0 % 4 == 0) && (z_col1 < 0 || z_col1 % 4 == 0) &&
+                     aligned(x) && aligned(z) && aligned(bias0) && aligned(bias1) && aligned(y0) && aligned(y1) &&
+                     aligned(weight);
+    if (!vec) return 3;
+    if (dtype == 0)
+        gated_add_norm_vec_kernel<float><<<n, S32_THREADS, 0, stream>>>((float*)out, x, z, z_stride, z_col0, z_col1, bias0, bias1,
+                                                                        y0, y0_stride, y1, y1_stride, weight, hidden, eps, offset);
+    else
+        gated_add_norm_vec_kernel<bf16><<<n, S32_THREADS, 0, stream>>>((bf16*)out, x, z, z_stride, z_col0, z_col1, bias0, bias1,
+                                                                       y0, y0_stride, y1, y1_stride, weight, hidden, eps, offset);
     LLMS_LAUNCH_CHECK();
 }
 

@@ -775,9 +775,8 @@ def rmsnorm32(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: flo
     return out
 
 
-def gated_add(x: torch.Tensor, branches: list, gate_products: torch.Tensor | None = None) -> torch.Tensor:
-    """x += sum over up to two branches of g * y, in place, all float32.  A branch is (y [N, hidden], column, bias):
-    g = sigmoid(gate_products[:, column : column + hidden] + bias) where `column` is not None, else 1."""
+def _gated_branches(x: torch.Tensor, branches: list, gate_products: torch.Tensor | None):
+    """Checks the operands of a gated sum; returns (device, z stride, [(y, column or -1, bias)] * 2)."""
     ys = [b for b in branches if b is not None]
     if not 1 <= len(ys) <= 2:
         raise ValueError("one or two branches")
@@ -803,6 +802,14 @@ def gated_add(x: torch.Tensor, branches: list, gate_products: torch.Tensor | Non
                 if bias is not None:
                     _f32(bias, "bias", hidden)
         args.append((y, -1 if column is None else column, bias if column is not None else None))
+    return dev, z_stride, args
+
+
+def gated_add(x: torch.Tensor, branches: list, gate_products: torch.Tensor | None = None) -> torch.Tensor:
+    """x += sum over up to two branches of g * y, in place, all float32.  A branch is (y [N, hidden], column, bias):
+    g = sigmoid(gate_products[:, column : column + hidden] + bias) where `column` is not None, else 1."""
+    dev, z_stride, args = _gated_branches(x, branches, gate_products)
+    n, hidden = x.shape
     if n == 0:
         return x
     (y0, c0, b0), (y1, c1, b1) = args
@@ -813,6 +820,39 @@ def gated_add(x: torch.Tensor, branches: list, gate_products: torch.Tensor | Non
     return x
 
 
+# Up to this many rows the sum and the norm are one kernel (a launch less in a step that is a chain of launches);
+# measured at 2,048 rows of 2,048: one kernel that walks a row in two turns 4 % of a prompt step slower than two.
+GATED_ADD_NORM_ROWS = 256
+
+
+def gated_add_norm(out: torch.Tensor, x: torch.Tensor, branches: list, gate_products: torch.Tensor | None,
+                   weight: torch.Tensor, eps: float, offset: float = 0.0) -> torch.Tensor:
+    """`gated_add(x, branches, gate_products)` and `rmsnorm32(out, x, weight, eps, offset)` of the summed rows, in
+    one kernel where the sizes allow (rows of a multiple of 4 up to 8,192), else one after the other."""
+    dev, z_stride, args = _gated_branches(x, branches, gate_products)
+    n, hidden = x.shape
+    _rows(out, "out", hidden)
+    _f32(weight, "weight", hidden)
+    if out.shape[0] != n:
+        raise ValueError("out and x differ in rows")
+    if n == 0:
+        return out
+    (y0, c0, b0), (y1, c1, b1) = args
+    if n > GATED_ADD_NORM_ROWS:  # many rows fill the chip either way, and two kernels that each read a row at once are faster
+        gated_add(x, branches, gate_products)
+        return rmsnorm32(out, x, weight, eps, offset)
+    status = load("stream32").llms_gated_add_norm(
+        c_int(_code(out)), _ptr(out), _ptr(x), _ptr(gate_products), c_int(z_stride), c_int(c0), c_int(c1), _ptr(b0),
+        _ptr(b1), _ptr(y0), c_int(y0.stride(0) if y0 is not None else 0), _ptr(y1),
+        c_int(y1.stride(0) if y1 is not None else 0), _ptr(weight), c_float(eps), c_float(offset), c_int(n),
+        c_int(hidden), _stream(dev))
+    if status == 3:  # sizes the fused kernel does not take
+        gated_add(x, branches, gate_products)
+        return rmsnorm32(out, x, weight, eps, offset)
+    _check(status, "gated_add_norm")
+    return out
+
+
 # ------------------------------------------------------------------------------ attention from chosen ingredients
 
 
@@ -821,12 +861,15 @@ def conv_store(q_out: torch.Tensor, proj: torch.Tensor, *, cq: int, k_heads: int
                state_slots: torch.Tensor | None = None, token_seq: torch.Tensor | None = None,
                positions: torch.Tensor | None = None, cu_seqlens: torch.Tensor | None = None,
                slots: torch.Tensor | None = None, k_pool: torch.Tensor | None = None,
-               v_pool: torch.Tensor | None = None, block_size: int = 0) -> torch.Tensor:
+               v_pool: torch.Tensor | None = None, block_size: int = 0, update_state: bool = False,
+               context_lens: torch.Tensor | None = None) -> torch.Tensor:
     """proj float32 [N, cq + k_heads*dk + v_heads*dv] (what the stacked q, k, v projection gave), optionally through a
     causal convolution per channel (`taps_w` float32 [channels, taps], `state` float32 [slots, taps-1, channels]: a
     ring of each request's last projected rows, indexed by position), rounded once: queries to q_out [N, cq], keys
-    and values to the tokens' cache slots (`slots`; None: nothing is stored)."""
-    dev = _dev(q_out, proj, taps_w, state, state_slots, token_seq, positions, cu_seqlens, slots, k_pool, v_pool)
+    and values to the tokens' cache slots (`slots`; None: nothing is stored).  `update_state` (only where every
+    request of the step brings exactly one token; `context_lens` [B] says which requests are padding): the ring takes
+    each token's projected row in the same kernel, so `conv_state` need not run."""
+    dev = _dev(q_out, proj, taps_w, state, state_slots, token_seq, positions, cu_seqlens, slots, k_pool, v_pool, context_lens)
     n = proj.shape[0]
     channels = cq + k_heads * dk + v_heads * dv
     if proj.dim() != 2 or proj.dtype != torch.float32 or proj.stride(1) != 1 or proj.shape[1] != channels:
@@ -858,6 +901,11 @@ def conv_store(q_out: torch.Tensor, proj: torch.Tensor, *, cq: int, k_heads: int
             raise ValueError(f"v_pool shape {tuple(v_pool.shape)} is not [pages,{v_heads},{dv},{block_size}]")
         if k_pool.dtype != q_out.dtype or v_pool.dtype != q_out.dtype:
             raise ValueError("pools and q_out differ in dtype")
+    fused_state = bool(update_state and taps > 1)
+    if fused_state:
+        if cu_seqlens.numel() - 1 != n:
+            raise ValueError("update_state needs every request to bring exactly one token")
+        _i32(context_lens, "context_lens", n)
     if n == 0:
         return q_out
     _check(load("attention_composed").llms_conv_store(
@@ -865,7 +913,8 @@ def conv_store(q_out: torch.Tensor, proj: torch.Tensor, *, cq: int, k_heads: int
         c_int(taps), _ptr(state), ctypes.c_size_t(state.stride(0) if state is not None else 0), _ptr(state_slots),
         _ptr(token_seq), _ptr(positions), _ptr(cu_seqlens), _ptr(slots), _ptr(k_pool), _ptr(v_pool), c_int(n), c_int(cq),
         c_int(k_heads * dk), c_int(v_heads * dv), c_int(k_heads), c_int(dk), c_int(v_heads), c_int(dv),
-        c_int(block_size), _stream(dev)), "conv_store")
+        c_int(block_size), _ptr(state if fused_state else None), _ptr(context_lens if fused_state else None),
+        _stream(dev)), "conv_store")
     return q_out
 
 
@@ -1029,7 +1078,7 @@ def attend_composed_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tenso
     if not (shares > 1 and talk is not None):
         shares = 1
     else:
-        shares = min(int(shares), 64)
+        shares = min(int(shares), 16)
         ws_stats = torch.empty((q.shape[0], heads, shares, 2), dtype=torch.float32, device=dev)
         ws_o = torch.empty((shares, q.shape[0], heads * dv), dtype=torch.float32, device=dev)
     _check(load("attention_composed_mfma").llms_attend_composed_mfma(

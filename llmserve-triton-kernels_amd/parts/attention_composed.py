@@ -160,13 +160,15 @@ class ComposedAttention(Mixer):
         proj = projected if projected is not None else linear(x, self.qkv_weight, out_dtype=torch.float32)
         q = torch.empty((proj.shape[0], self.cq), dtype=x.dtype, device=x.device)
         conv, taps = self.taps > 1, self.taps > 0  # (one tap is a factor per channel and needs no state)
+        single = conv and batch.max_count == 1 and batch.num_seqs == proj.shape[0]  # every request brings one token
         ops.conv_store(q, proj, cq=self.cq, k_heads=kv * self.maps, dk=dk, v_heads=kv, dv=dv,
                        taps_w=self.taps_w if taps else None,
                        state=state.state if conv else None, state_slots=batch.state_slots if conv else None,
                        token_seq=batch.token_seq if taps else None, positions=batch.positions if taps else None,
                        cu_seqlens=batch.cu_seqlens if taps else None, slots=view.slots if paged.store else None,
-                       k_pool=paged.k_pool, v_pool=paged.v_pool, block_size=paged.block_size)
-        if conv:
+                       k_pool=paged.k_pool, v_pool=paged.v_pool, block_size=paged.block_size, update_state=single,
+                       context_lens=batch.context_lens if single else None)
+        if conv and not single:
             ops.conv_state(state.state, proj, batch.state_slots, batch.cu_seqlens, batch.context_lens)
         out = torch.empty((proj.shape[0], heads * dv), dtype=x.dtype, device=x.device)
         self.attend(out, q, paged, view, batch)

@@ -18,7 +18,7 @@ import torch
 
 from ..ops import library as ops
 from .linear import linear
-from .registry import ADDED_IN_PLACE, Block, DeferredNorm, register_block
+from .registry import ADDED_IN_PLACE, Block, DeferredNorm, GatedSum, register_block
 
 
 @register_block("prenorm")
@@ -88,9 +88,10 @@ class ParallelBlock(Block):
         return one, (0 if zm is not None else None), (0 if zf is not None else None), None
 
     def forward(self, x, delta, batch, cache):
-        if delta is not None or x.dtype != torch.float32:
-            raise ValueError("the parallel arrangement keeps a closed 32-bit residual stream")
-        h = self.norm.forward(x)
+        if x.dtype != torch.float32:
+            raise ValueError("the parallel arrangement keeps a 32-bit residual stream")
+        # (the layer before may have left its gated sum open: this layer's norm closes it in its own kernel)
+        h = self.norm.add_norm(x, delta)
         z, col_m, col_f, projected = self._gate_products(h)
         a = self.mixer.forward(h, batch, cache) if projected is None else self.mixer.forward(h, batch, cache, projected=projected)
         f = self.feed_forward.forward(h)
@@ -98,6 +99,9 @@ class ParallelBlock(Block):
         for y, col, gate in ((a, col_m, self.mixer_gate), (f, col_f, self.feed_forward_gate)):
             if y is not None:
                 branches.append((y if y.dtype == torch.float32 else y.float(), col, gate.bias))
-        if branches:
-            ops.gated_add(x, branches, z)
+        if not branches:
+            return x, None
+        if getattr(self.norm, "closes_gated_sums", False):  # left open for the next norm (the next layer's, or the last)
+            return x, GatedSum(branches, z)
+        ops.gated_add(x, branches, z)
         return x, None

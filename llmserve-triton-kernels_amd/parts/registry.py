@@ -102,6 +102,16 @@ class PartialSums:
         return acc.to(self.dtype)
 
 
+@dataclass
+class GatedSum:
+    """A residual sum that is still open: x += sum over `branches` of g * y, with (y, column, bias) per branch and
+    the gates' products in `gate_products` (the operands of ops.gated_add).  An arrangement with a 32-bit stream
+    hands it on in the place of `delta`; a norm that knows it closes the sum in its own kernel (`add_norm`)."""
+
+    branches: list
+    gate_products: "torch.Tensor | None"
+
+
 def as_tensor(delta):
     """`delta` as a tensor in the model's dtype (None stays None)."""
     return delta.total() if isinstance(delta, PartialSums) else delta

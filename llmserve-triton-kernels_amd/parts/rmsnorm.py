@@ -6,7 +6,7 @@ from __future__ import annotations
 import torch
 
 from ..ops import library as ops
-from .registry import PartialSums, Norm, register_norm
+from .registry import GatedSum, PartialSums, Norm, register_norm
 from .spec import ParamInfo
 
 
@@ -56,6 +56,7 @@ class RMSNorm32(Norm):
     no `rms_params`: the products that norm their rows on the way in round where this norm does not."""
 
     graph_safe = True
+    closes_gated_sums = True  # `add_norm` and `norm_rows` take a `GatedSum` in the place of delta
 
     def __init__(self, spec, ctx):
         super().__init__(spec, ctx)
@@ -79,13 +80,19 @@ class RMSNorm32(Norm):
         return ops.rmsnorm32(out, self._stream(x), self.weight, self.eps, self.offset)
 
     def add_norm(self, residual, delta):
-        if delta is not None:
-            raise ValueError("a 32-bit residual stream is summed by the arrangement, not by its norm")
-        return self.forward(residual)
+        """`delta`: None, or the open gated sum of the layer before (closed here, in the norm's own kernel)."""
+        if delta is None:
+            return self.forward(residual)
+        if not isinstance(delta, GatedSum) or residual.dtype != torch.float32:
+            raise ValueError("a 32-bit residual stream takes an open gated sum or nothing")
+        out = torch.empty(residual.shape, dtype=self.ctx.dtype, device=residual.device)
+        return ops.gated_add_norm(out, residual, delta.branches, delta.gate_products, self.weight, self.eps, self.offset)
 
     def norm_rows(self, x, delta, rows):
-        if delta is not None:
-            raise ValueError("a 32-bit residual stream is summed by the arrangement, not by its norm")
+        if delta is not None:  # (few rows are wanted, but every row's sum is closed: the stream is the caller's)
+            if not isinstance(delta, GatedSum) or x.dtype != torch.float32:
+                raise ValueError("a 32-bit residual stream takes an open gated sum or nothing")
+            ops.gated_add(x, delta.branches, delta.gate_products)
         out = torch.empty((rows.numel(), self.hidden), dtype=self.ctx.dtype, device=x.device)
         return ops.rmsnorm32(out, self._stream(x), self.weight, self.eps, self.offset, rows=rows)
 

@@ -62,6 +62,18 @@ def test_scaled_embedding_norm_and_gated_sum(dtype, hidden):
     ref = stream.double() + a.double() + torch.sigmoid(z[:, hidden:].double() + b2.double()) * f.double()
     got = ops.gated_add(stream.clone().to(DEV), [(a.to(DEV), None, None), (f.to(DEV), hidden, b2.to(DEV))], z.to(DEV))
     close(got, ref, torch.float32, "a plain branch beside a gated one")
+    # the sum and the norm of the summed rows in one kernel (rows that are no multiple of 4: one after the other)
+    summed = stream.clone().to(DEV)
+    out = ops.gated_add_norm(torch.empty(6, hidden, dtype=dtype, device=DEV), summed,
+                             [(a.to(DEV), None, None), (f.to(DEV), hidden, b2.to(DEV))], z.to(DEV), w.to(DEV), 1e-5, 1.0)
+    close(summed, ref, torch.float32, "the summed rows")
+    close(out, pd.norm_zero_centred(ref, w.double(), 1e-5), dtype, "their norm")
+    many = ops.GATED_ADD_NORM_ROWS + 3  # beyond this many rows: two kernels
+    big, ya = rnd(many, hidden, seed=9).float(), rnd(many, hidden, seed=10).float()
+    summed = big.clone().to(DEV)
+    out = ops.gated_add_norm(torch.empty(many, hidden, dtype=dtype, device=DEV), summed, [(ya.to(DEV), None, None)], None,
+                             w.to(DEV), 1e-5, 1.0)
+    close(out, pd.norm_zero_centred(big.double() + ya.double(), w.double(), 1e-5), dtype, "many rows")
 
 
 # ------------------------------------------------------------------------------ convolution, state and cache store
