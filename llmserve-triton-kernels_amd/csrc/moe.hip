@@ -1,0 +1,181 @@
+// Routing for a feed-forward of many small experts, of which each token uses `top`.
+//   moe_router    z = W_router h in 32-bit, s = sigmoid(z) (or softmax is not offered: the scores are independent),
+//                 the `top` largest (the lower expert wins a tie), in descending order; weight = score or
+//                 score / sum of the chosen scores
+//   moe_rank      for expert e: how many (token, choice) pairs chose it, and each such pair's rank among them in the
+//                 order of the pairs (so the sorted order is stable and the same whatever runs beside it)
+//   moe_offsets   seg[e] = pairs of all experts before e, tile_start[e] = tiles of `tile` rows of all experts before e
+//   moe_scatter   rows sorted by expert: xs[seg[e] + rank] = weight * h[token] (the weight multiplies the expert's
+//                 input), rounded to T; place[pair] = that row
+//   moe_combine   y[n] = sum over the token's choices, in their order, of the experts' results rows (32-bit)
+// A pair is p = token * top + choice.
+#include "common.h"
+
+#define MOE_THREADS 256
+#define MOE_MAX_TOP 16
+
+template <typename T>
+__global__ __launch_bounds__(MOE_THREADS) void moe_router_kernel(
+    int* __restrict__ chosen, float* __restrict__ weight, const T* __restrict__ h, const T* __restrict__ w_router,
+    int hidden, int experts, int top, int renormalize) {
+    extern __shared__ float score[];  // experts
+    const int n = blockIdx.x, lane = threadIdx.x % LLMS_WAVE, wave = threadIdx.x / LLMS_WAVE;
+    const T* row = h + (size_t)n * hidden;
+    for (int e = wave; e < experts; e += MOE_THREADS / LLMS_WAVE) {
+        const T* wr = w_router + (size_t)e * hidden;
+        float dot = 0.f;
+        for (int c = lane; c < hidden; c += LLMS_WAVE) dot = fmaf(to_f32(row[c]), to_f32(wr[c]), dot);
+        dot = wave_sum(dot);
+        if (lane == 0) score[e] = 1.f / (1.f + expf(-dot));
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    float picked[MOE_MAX_TOP];
+    int which[MOE_MAX_TOP];
+    float sum = 0.f;
+    for (int k = 0; k < top; ++k) {
+        float best = -1.f;  // (scores are in (0, 1); a taken expert is marked -2)
+        int at = 0x7fffffff;
+        for (int e = lane; e < experts; e += LLMS_WAVE) {
+            const float s = score[e];
+            if (s > best) {
+                best = s;
+                at = e;
+            }
+        }
+#pragma unroll
+        for (int o = LLMS_WAVE / 2; o > 0; o >>= 1) {
+            const float ob = __shfl_xor(best, o, LLMS_WAVE);
+            const int oa = __shfl_xor(at, o, LLMS_WAVE);
+            if (ob > best || (ob == best && oa < at)) {
+                best = ob;
+                at = oa;
+            }
+        }
+        picked[k] = best;
+        which[k] = at;
+        sum += best;
+        if (lane == 0) score[at] = -2.f;
+        __builtin_amdgcn_s_waitcnt(0);
+        __builtin_amdgcn_wave_barrier();
+    }
+    if (lane == 0)
+        for (int k = 0; k < top; ++k) {
+            chosen[(size_t)n * top + k] = which[k];
+            weight[(size_t)n * top + k] = renormalize ? picked[k] / sum : picked[k];
+        }
+}
+
+// grid: experts.  One workgroup walks all pairs in order, 256 at a time.
+__global__ __launch_bounds__(MOE_THREADS) void moe_rank_kernel(int* __restrict__ count, int* __restrict__ rank,
+                                                               const int* __restrict__ chosen, int pairs) {
+    __shared__ int wave_total[MOE_THREADS / LLMS_WAVE];
+    const int e = blockIdx.x, lane = threadIdx.x % LLMS_WAVE, wave = threadIdx.x / LLMS_WAVE;
+    int base = 0;
+    for (int p0 = 0; p0 < pairs; p0 += MOE_THREADS) {
+        const int p = p0 + threadIdx.x;
+        const bool mine = p < pairs && chosen[p] == e;
+        const unsigned long long votes = __ballot(mine);
+        const int before = __popcll(votes & ((1ull << lane) - 1ull));
+        if (lane == 0) wave_total[wave] = __popcll(votes);
+        __syncthreads();
+        int ahead = 0, all = 0;
+#pragma unroll
+        for (int w = 0; w < MOE_THREADS / LLMS_WAVE; ++w) {
+            ahead += w < wave ? wave_total[w] : 0;
+            all += wave_total[w];
+        }
+        if (mine) rank[p] = base + ahead + before;
+        base += all;
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) count[e] = base;
+}
+
+// one workgroup of one thread's work: experts are few
+__global__ void moe_offsets_kernel(int* __restrict__ seg, int* __restrict__ tile_start, const int* __restrict__ count,
+                                   int experts, int tile) {
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    int rows = 0, tiles = 0;
+    for (int e = 0; e < experts; ++e) {
+        seg[e] = rows;
+        tile_start[e] = tiles;
+        rows += count[e];
+        tiles += (count[e] + tile - 1) / tile;
+    }
+    seg[experts] = rows;
+    tile_start[experts] = tiles;
+}
+
+// grid: pairs
+template <typename T>
+__global__ __launch_bounds__(MOE_THREADS) void moe_scatter_kernel(
+    T* __restrict__ xs, int* __restrict__ place, const T* __restrict__ h, const int* __restrict__ chosen,
+    const float* __restrict__ weight, const int* __restrict__ rank, const int* __restrict__ seg, int hidden, int top) {
+    const int p = blockIdx.x, n = p / top;
+    const int dest = seg[chosen[p]] + rank[p];
+    const float wgt = weight[p];
+    if (threadIdx.x == 0) place[p] = dest;
+    const T* src = h + (size_t)n * hidden;
+    T* dst = xs + (size_t)dest * hidden;
+    for (int c = threadIdx.x; c < hidden; c += MOE_THREADS) dst[c] = from_f32<T>(wgt * to_f32(src[c]));
+}
+
+// grid: tokens
+__global__ __launch_bounds__(MOE_THREADS) void moe_combine_kernel(float* __restrict__ y, const float* __restrict__ rows,
+                                                                  const int* __restrict__ place, int hidden, int top) {
+    const int n = blockIdx.x;
+    for (int c = threadIdx.x; c < hidden; c += MOE_THREADS) {
+        float v = 0.f;
+        for (int k = 0; k < top; ++k) v += rows[(size_t)place[(size_t)n * top + k] * hidden + c];
+        y[(size_t)n * hidden + c] = v;
+    }
+}
+
+extern "C" {
+
+int llms_moe_router(int dtype, int* chosen, float* weight, const void* h, const void* w_router, int n, int hidden, int experts,
+                    int top, int renormalize, hipStream_t stream) {
+    LLMS_REQUIRE(n > 0 && hidden > 0 && experts > 0, "moe_router: sizes must be positive");
+    LLMS_REQUIRE(top >= 1 && top <= MOE_MAX_TOP && top <= experts, "moe_router: 1 to 16 choices, no more than there are experts");
+    LLMS_REQUIRE(experts <= 8192, "moe_router: up to 8,192 experts");
+    LLMS_REQUIRE(dtype == 0 || dtype == 1, "moe_router: dtype must be 0 (float32) or 1 (bfloat16)");
+    const size_t lds = (size_t)experts * sizeof(float);
+    if (dtype == 0)
+        moe_router_kernel<float><<<n, MOE_THREADS, lds, stream>>>(chosen, weight, (const float*)h, (const float*)w_router, hidden,
+                                                                  experts, top, renormalize);
+    else
+        moe_router_kernel<bf16><<<n, MOE_THREADS, lds, stream>>>(chosen, weight, (const bf16*)h, (const bf16*)w_router, hidden,
+                                                                 experts, top, renormalize);
+    LLMS_LAUNCH_CHECK();
+}
+
+// count [E], rank [pairs], seg [E + 1], tile_start [E + 1]
+int llms_moe_sort(int* count, int* rank, int* seg, int* tile_start, const int* chosen, int pairs, int experts, int tile,
+                  hipStream_t stream) {
+    LLMS_REQUIRE(pairs > 0 && experts > 0 && tile > 0, "moe_sort: sizes must be positive");
+    moe_rank_kernel<<<experts, MOE_THREADS, 0, stream>>>(count, rank, chosen, pairs);
+    moe_offsets_kernel<<<1, 64, 0, stream>>>(seg, tile_start, count, experts, tile);
+    LLMS_LAUNCH_CHECK();
+}
+
+int llms_moe_scatter(int dtype, void* xs, int* place, const void* h, const int* chosen, const float* weight, const int* rank,
+                     const int* seg, int pairs, int hidden, int top, hipStream_t stream) {
+    LLMS_REQUIRE(pairs > 0 && hidden > 0 && top > 0, "moe_scatter: sizes must be positive");
+    LLMS_REQUIRE(dtype == 0 || dtype == 1, "moe_scatter: dtype must be 0 (float32) or 1 (bfloat16)");
+    if (dtype == 0)
+        moe_scatter_kernel<float><<<pairs, MOE_THREADS, 0, stream>>>((float*)xs, place, (const float*)h, chosen, weight, rank, seg,
+                                                                     hidden, top);
+    else
+        moe_scatter_kernel<bf16><<<pairs, MOE_THREADS, 0, stream>>>((bf16*)xs, place, (const bf16*)h, chosen, weight, rank, seg,
+                                                                    hidden, top);
+    LLMS_LAUNCH_CHECK();
+}
+
+int llms_moe_combine(float* y, const float* rows, const int* place, int n, int hidden, int top, hipStream_t stream) {
+    LLMS_REQUIRE(n > 0 && hidden > 0 && top > 0, "moe_combine: sizes must be positive");
+    moe_combine_kernel<<<n, MOE_THREADS, 0, stream>>>(y, rows, place, hidden, top);
+    LLMS_LAUNCH_CHECK();
+}
+
+}  // extern "C"

@@ -4,6 +4,10 @@
 //   gated_add        x[n] += sum over branches b of g_b * y_b[n]                    (all float)
 //                    g_b = sigmoid(z_b[n] + bias_b) where the branch has a gate, else 1
 //   gated_add_norm   the same sum and, in the same kernel, the norm of the summed row for the next layer
+//   streams_norm     a residual stream of S parallel copies (S = 1: the plain residual sum).  With the result y of
+//                    the sublayer before and its coefficients, new_t = sum_s mix[s, t] x_s + out[t] y for all t at
+//                    once; u = sum_t read[t] new_t; out = (u - mean) / sqrt(var + eps) * w (layer norm, no bias; the
+//                    variance is the mean squared deviation).                       (x, y, coefficients float; out T)
 // T is float or bfloat16.  One workgroup per row; every reduction has an order fixed by the sizes alone.
 #include "common.h"
 
@@ -190,6 +194,71 @@ __global__ __launch_bounds__(S32_THREADS) void gated_add_kernel(float* __restric
     }
 }
 
+#define STREAMS_MAX 8
+
+// One workgroup a row.  x_src is [N, S, hidden] (stream stride `hidden`) or, with src_broadcast, [N, hidden] read as
+// S equal copies; x_dst (may be x_src itself: every thread reads all of a column's streams before it writes them) takes
+// the new streams when `store`.  `y` null: nothing is added and the streams pass as they are.  `read` null: the plain
+// sum of the streams.  `rows`: only these rows are worked out (out[r] from row rows[r]).  Dynamic LDS: hidden floats.
+template <typename T>
+__global__ __launch_bounds__(S32_THREADS) void streams_norm_kernel(
+    T* __restrict__ out, float* x_dst, const float* x_src, int src_broadcast, const float* __restrict__ y,
+    const float* __restrict__ mix, const float* __restrict__ wout, const float* __restrict__ read,
+    const float* __restrict__ weight, const int* __restrict__ rows, int streams, int hidden, float eps, int store) {
+    extern __shared__ float u_row[];
+    __shared__ float red[16];
+    __shared__ float coef[STREAMS_MAX * STREAMS_MAX + 2 * STREAMS_MAX];
+    const int r = blockIdx.x, n = rows ? rows[r] : r, S = streams;
+    for (int i = threadIdx.x; i < S * S + 2 * S; i += S32_THREADS) {
+        float v;
+        if (i < S * S) v = mix ? mix[i] : (i / S == i % S ? 1.f : 0.f);
+        else if (i < S * S + S) v = wout ? wout[i - S * S] : 1.f;
+        else v = read ? read[i - S * S - S] : 1.f;
+        coef[i] = v;
+    }
+    __syncthreads();
+    const float* cm = coef;
+    const float* co = coef + S * S;
+    const float* cr = co + S;
+    const float* src = x_src + (size_t)n * hidden * (src_broadcast ? 1 : S);
+    float* dst = x_dst + (size_t)n * hidden * S;
+    float total = 0.f;
+    for (int c = threadIdx.x; c < hidden; c += S32_THREADS) {
+        float xs[STREAMS_MAX];
+#pragma unroll
+        for (int s = 0; s < STREAMS_MAX; ++s) xs[s] = s < S ? src[src_broadcast ? c : (size_t)s * hidden + c] : 0.f;
+        const float yv = y ? y[(size_t)n * hidden + c] : 0.f;
+        float u = 0.f;
+#pragma unroll
+        for (int t = 0; t < STREAMS_MAX; ++t) {
+            if (t < S) {
+                float v = xs[t];
+                if (y) {
+                    v = 0.f;
+#pragma unroll
+                    for (int s = 0; s < STREAMS_MAX; ++s)
+                        if (s < S) v = fmaf(cm[s * S + t], xs[s], v);
+                    v = fmaf(co[t], yv, v);
+                }
+                if (store) dst[(size_t)t * hidden + c] = v;
+                u = fmaf(cr[t], v, u);
+            }
+        }
+        u_row[c] = u;
+        total += u;
+    }
+    const float mean = block_sum(total, red) / (float)hidden;
+    float dev2 = 0.f;
+    for (int c = threadIdx.x; c < hidden; c += S32_THREADS) {
+        const float d = u_row[c] - mean;
+        dev2 = fmaf(d, d, dev2);
+    }
+    const float inv = 1.0f / sqrtf(block_sum(dev2, red) / (float)hidden + eps);
+    if (!out) return;
+    T* orow = out + (size_t)r * hidden;
+    for (int c = threadIdx.x; c < hidden; c += S32_THREADS) orow[c] = from_f32<T>((u_row[c] - mean) * inv * weight[c]);
+}
+
 extern "C" {
 
 int llms_embed_scale(int dtype, float* out, const void* table, const int* ids, int n, int hidden, int vocab, float scale,
@@ -265,6 +334,28 @@ int llms_gated_add_norm(int dtype, void* out, float* x, const float* z, int z_st
     else
         gated_add_norm_vec_kernel<bf16><<<n, S32_THREADS, 0, stream>>>((bf16*)out, x, z, z_stride, z_col0, z_col1, bias0, bias1,
                                                                        y0, y0_stride, y1, y1_stride, weight, hidden, eps, offset);
+    LLMS_LAUNCH_CHECK();
+}
+
+int llms_streams_norm(int dtype, void* out, float* x_dst, const float* x_src, int src_broadcast, const float* y,
+                      const float* mix, const float* wout, const float* read, const float* weight, const int* rows,
+                      int n_out, int streams, int hidden, float eps, int store, hipStream_t stream) {
+    LLMS_REQUIRE(n_out > 0 && hidden > 0, "streams_norm: sizes must be positive");
+    LLMS_REQUIRE(streams >= 1 && streams <= STREAMS_MAX, "streams_norm: 1 to 8 streams");
+    LLMS_REQUIRE(dtype == 0 || dtype == 1, "streams_norm: dtype must be 0 (float32) or 1 (bfloat16)");
+    LLMS_REQUIRE(x_src && (x_dst || !store) && (weight || !out), "streams_norm: a needed operand is missing");
+    LLMS_REQUIRE((size_t)hidden * 4 <= 96 * 1024, "streams_norm: a row of up to 24,576 elements");
+    const size_t lds = (size_t)hidden * sizeof(float);
+    if (lds > 32 * 1024) {
+        const void* kernel = dtype == 0 ? (const void*)streams_norm_kernel<float> : (const void*)streams_norm_kernel<bf16>;
+        LLMS_HIP_CHECK(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    }
+    if (dtype == 0)
+        streams_norm_kernel<float><<<n_out, S32_THREADS, lds, stream>>>((float*)out, x_dst, x_src, src_broadcast, y, mix, wout,
+                                                                        read, weight, rows, streams, hidden, eps, store);
+    else
+        streams_norm_kernel<bf16><<<n_out, S32_THREADS, lds, stream>>>((bf16*)out, x_dst, x_src, src_broadcast, y, mix, wout,
+                                                                       read, weight, rows, streams, hidden, eps, store);
     LLMS_LAUNCH_CHECK();
 }
 

@@ -1120,3 +1120,311 @@ def sample_rows(out: torch.Tensor, logits: torch.Tensor, temperature: torch.Tens
         _ptr(out), _ptr(logits), c_int(logits.stride(0)), c_int(r), c_int(v), _ptr(temperature), _ptr(top_k),
         _ptr(top_p), _ptr(uniform), _stream(dev)), "sample_rows")
     return out
+
+
+# ------------------------------------------------------------------------------ streams of residuals, layer norm
+
+STREAMS_MAX = 8
+
+
+def streams_norm(out: torch.Tensor | None, x: torch.Tensor, weight: torch.Tensor | None, eps: float, *,
+                 source: torch.Tensor | None = None, y: torch.Tensor | None = None, mix: torch.Tensor | None = None,
+                 write: torch.Tensor | None = None, read: torch.Tensor | None = None,
+                 rows: torch.Tensor | None = None) -> torch.Tensor | None:
+    """A residual stream of S copies x [N, S, hidden] (float32), in one kernel:
+    with `y` [N, hidden] the streams become new_t = sum_s mix[s, t] x_s + write[t] y, all at once (stored into x
+    unless `rows` picks rows); u = sum_t read[t] new_t (`read` None: the plain sum); out = layer norm of u with
+    `weight`, no bias, rounded once to out's dtype.  `source` [N, hidden]: the streams are read as S copies of it
+    (and stored into x).  `rows`: out[r] is worked out from row rows[r], nothing is stored.  `out` None: only the
+    streams are brought up to date."""
+    dev = _dev(out, x, weight, source, y, mix, write, read, rows)
+    if x.dim() != 3 or x.dtype != torch.float32 or not x.is_contiguous():
+        raise ValueError(f"x must be a contiguous float32 [N, S, hidden] tensor, got {tuple(x.shape)} {x.dtype}")
+    n, s, hidden = x.shape
+    if not 1 <= s <= STREAMS_MAX:
+        raise ValueError(f"1 to {STREAMS_MAX} streams, got {s}")
+    if hidden * 4 > 96 * 1024:
+        raise ValueError("rows of up to 24,576 elements")
+    for t, name, numel in ((mix, "mix", s * s), (write, "write", s), (read, "read", s)):
+        if t is not None:
+            _f32(t, name, numel)
+    if (mix is None) != (write is None) or (y is None and mix is not None):
+        raise ValueError("mix and write come together, with y")
+    if y is not None:
+        _f32(y, "y", n * hidden)
+    if source is not None:
+        _f32(source, "source", n * hidden)
+    store = rows is None
+    if rows is not None:
+        _i32(rows, "rows")
+        n_out = rows.numel()
+    else:
+        n_out = n
+    if out is not None:
+        _rows(out, "out", hidden)
+        if out.shape[0] != n_out:
+            raise ValueError(f"out has {out.shape[0]} rows, expected {n_out}")
+        _f32(weight, "weight", hidden)
+    elif not store or (y is None and source is None):
+        raise ValueError("nothing to do: no output and nothing to store")
+    if n_out == 0:
+        return out
+    src = source if source is not None else x
+    _check(load("stream32").llms_streams_norm(
+        c_int(_code(out) if out is not None else 0), _ptr(out), _ptr(x), _ptr(src), c_int(source is not None), _ptr(y),
+        _ptr(mix), _ptr(write), _ptr(read), _ptr(weight), _ptr(rows), c_int(n_out), c_int(s), c_int(hidden), c_float(eps),
+        c_int(1 if store and (y is not None or source is not None) else 0), _stream(dev)), "streams_norm")
+    return out
+
+
+# ------------------------------------------------------------------------------ attention through a latent
+
+
+def _latent_rotation(freq: torch.Tensor | None, dr: int) -> int:
+    if freq is None:
+        return 0
+    _f32(freq, "freq")
+    dims = 2 * freq.numel()
+    if dims > dr:
+        raise ValueError(f"{dims} turned dimensions in a part of {dr}")
+    return dims
+
+
+def latent_prepare(z: torch.Tensor, *, col_q: int, q_rank: int, col_c: int | None, r: int, dr: int, wq: torch.Tensor,
+                   wc: torch.Tensor | None, freq: torch.Tensor | None, positions: torch.Tensor, eps: float,
+                   cq: torch.Tensor, pool: torch.Tensor | None = None, slots: torch.Tensor | None = None) -> torch.Tensor:
+    """From the 32-bit input products z [N, columns]: cq [N, q_rank] = z[:, col_q:][:q_rank] over its root mean
+    square times wq; with `col_c`, the cache rows pool[slots[n]] = [z_c over its root mean square times wc ; the dr
+    columns behind it with their first 2 len(freq) dimensions turned by the token's position (pairs 2i, 2i+1)].
+    pool [pages, 1, block, r + dr] in the dtype of cq."""
+    dev = _dev(z, wq, wc, freq, positions, cq, pool, slots)
+    if z.dim() != 2 or z.dtype != torch.float32 or z.stride(1) != 1:
+        raise ValueError("z must be a float32 matrix with unit inner stride")
+    n = z.shape[0]
+    _rows(cq, "cq", q_rank)
+    _f32(wq, "wq", q_rank)
+    _i32(positions, "positions", n)
+    dims = _latent_rotation(freq, dr)
+    if col_q < 0 or col_q + q_rank > z.shape[1]:
+        raise ValueError("the query latent's columns lie outside z")
+    if col_c is not None:
+        if col_c < 0 or col_c + r + dr > z.shape[1]:
+            raise ValueError("the latent's columns lie outside z")
+        _f32(wc, "wc", r)
+        if pool is None or slots is None or pool.dtype != cq.dtype or not pool.is_contiguous() or pool.shape[-1] != r + dr:
+            raise ValueError("a layer that keeps a latent needs its pool [.., r + dr] in cq's dtype and the tokens' slots")
+        _i32(slots, "slots", n)
+    if cq.shape[0] != n:
+        raise ValueError("cq and z differ in rows")
+    if n == 0:
+        return cq
+    _check(load("latent").llms_latent_prepare(
+        c_int(_code(cq)), _ptr(cq), _ptr(pool if col_c is not None else None), _ptr(z), c_int(z.stride(0)), c_int(col_q),
+        c_int(q_rank), c_int(-1 if col_c is None else col_c), c_int(r), c_int(dr), _ptr(wq), _ptr(wc), _ptr(freq), c_int(dims),
+        _ptr(positions), _ptr(slots if col_c is not None else None), c_float(eps), c_int(n), _stream(dev)), "latent_prepare")
+    return cq
+
+
+def latent_query(plain: torch.Tensor, folded: torch.Tensor, q: torch.Tensor, *, heads: int, dn: int, dr: int, r: int,
+                 freq: torch.Tensor | None, positions: torch.Tensor) -> None:
+    """q [N, heads * (dn + dr)] float32 -> plain [N, heads * dn] (the unrotated parts) and folded[n, h, r:] (the
+    rotated parts, turned); folded [N, heads * (r + dr)]."""
+    dev = _dev(plain, folded, q, freq, positions)
+    n = q.shape[0]
+    _f32(q, "q", n * heads * (dn + dr))
+    _rows(plain, "plain", heads * dn)
+    _rows(folded, "folded", heads * (r + dr))
+    _i32(positions, "positions", n)
+    if plain.dtype != folded.dtype or plain.shape[0] != n or folded.shape[0] != n:
+        raise ValueError("plain and folded share one dtype and q's rows")
+    dims = _latent_rotation(freq, dr)
+    if n == 0:
+        return
+    _check(load("latent").llms_latent_query(
+        c_int(_code(plain)), _ptr(plain), _ptr(folded), _ptr(q), c_int(heads), c_int(dn), c_int(dr), c_int(r), _ptr(freq),
+        c_int(dims), _ptr(positions), c_int(n), _stream(dev)), "latent_query")
+
+
+LATENT_ROW_MAX = 1024
+
+
+def attend_latent(out: torch.Tensor, q: torch.Tensor, pool: torch.Tensor, block_tables: torch.Tensor,
+                  token_seq: torch.Tensor, positions: torch.Tensor, context_lens: torch.Tensor, *, heads: int, r: int,
+                  dr: int, block_size: int, window: int, scale: float, table_rows: torch.Tensor | None = None) -> torch.Tensor:
+    """out[n, h] = sum_j softmax_j(scale q[n, h] . row_j) row_j[:r] over the cache rows j of token n's request with
+    0 <= position - j < window (window 0: every j <= position); q [N, heads * (r + dr)], out [N, heads * r], pool
+    [pages, 1, block, r + dr]."""
+    dev = _dev(out, q, pool, block_tables, token_seq, positions, context_lens, table_rows)
+    n = q.shape[0]
+    _rows(q, "q", heads * (r + dr))
+    _rows(out, "out", heads * r)
+    if out.shape[0] != n or out.dtype != q.dtype or pool.dtype != q.dtype:
+        raise ValueError("out, q and pool share one dtype; out and q their rows")
+    if not pool.is_contiguous() or pool.dim() != 4 or pool.shape[1] != 1 or pool.shape[2] != block_size or pool.shape[3] != r + dr:
+        raise ValueError(f"pool must be [pages, 1, {block_size}, {r + dr}], got {tuple(pool.shape)}")
+    if r + dr > LATENT_ROW_MAX:
+        raise ValueError(f"a cache row of up to {LATENT_ROW_MAX} numbers")
+    if block_tables.dtype != torch.int32 or block_tables.dim() != 2 or not block_tables.is_contiguous():
+        raise ValueError("block_tables must be a contiguous int32 matrix")
+    _i32(token_seq, "token_seq", n)
+    _i32(positions, "positions", n)
+    _i32(context_lens, "context_lens")
+    if table_rows is not None:
+        _i32(table_rows, "table_rows", context_lens.numel())
+    elif block_tables.shape[0] < context_lens.numel():
+        raise ValueError("fewer block tables than requests")
+    if window < 0:
+        raise ValueError("window must be >= 0")
+    if n == 0:
+        return out
+    _check(load("latent").llms_attend_latent(
+        c_int(_code(q)), _ptr(out), _ptr(q), _ptr(pool), _ptr(block_tables), c_int(block_tables.shape[1]), _ptr(table_rows),
+        _ptr(token_seq), _ptr(positions), _ptr(context_lens), c_int(n), c_int(heads), c_int(r), c_int(dr), c_int(block_size),
+        c_int(window), c_float(scale), _stream(dev)), "attend_latent")
+    return out
+
+
+# ------------------------------------------------------------------------------ products with a weight per group
+
+c_long = ctypes.c_long
+GROUPED_TILE = 64
+_EPILOGUES = {"plain": 0, "paired": 1, "gated": 2}
+
+
+def grouped_product(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, *, epilogue: str = "plain",
+                    segments: "tuple[torch.Tensor, torch.Tensor] | None" = None, gate: torch.Tensor | None = None,
+                    gate_column: int = 0, limit: float = 0.0) -> torch.Tensor:
+    """w [G, N, K].  Without `segments` every row meets every group: x [M, G, K] and out [M, G, N'] (views whose
+    last axis has unit stride; the strides of the other two are free), out[m, g] = x[m, g] w[g]^T.  With `segments`
+    = (seg [G + 1], tile_start [G + 1]) on the device, x [M, K] and out [M, N'] hold rows sorted by group, rows
+    seg[g] .. seg[g + 1] belonging to group g, and tile_start counts tiles of GROUPED_TILE rows.
+    Epilogues: "plain" (N' = N); "paired" (N' = N / 2: the weight's rows alternate between the two projections a, b of
+    a gated unit, out = min(a, limit) sigmoid(1.702 min(a, limit)) (clamp(b, +-limit) + 1)); "gated" (out times
+    sigmoid(gate[m, gate_column + g N + n]), gate float32 [M, columns])."""
+    dev = _dev(out, x, w, gate, *(segments or ()))
+    if w.dim() != 3 or not w.is_contiguous():
+        raise ValueError("w must be a contiguous [G, N, K] tensor")
+    g, n, k = w.shape
+    n_out = n // 2 if epilogue == "paired" else n
+    if epilogue not in _EPILOGUES or (epilogue == "paired" and n % 2):
+        raise ValueError(f"epilogue {epilogue!r} with {n} weight rows")
+    if x.dtype != w.dtype or (x.dtype, out.dtype) not in ((torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                                         (torch.bfloat16, torch.float32)):
+        raise ValueError(f"grouped_product does not take {x.dtype} x {w.dtype} -> {out.dtype}")
+    if segments is None:
+        if x.dim() != 3 or out.dim() != 3 or x.stride(2) != 1 or out.stride(2) != 1:
+            raise ValueError("x and out must be [M, G, .] views with unit inner stride")
+        if tuple(x.shape[1:]) != (g, k) or tuple(out.shape) != (x.shape[0], g, n_out):
+            raise ValueError(f"x {tuple(x.shape)} and out {tuple(out.shape)} do not fit w {tuple(w.shape)}")
+        m = x.shape[0]
+        x_ld, x_gs, out_ld, out_gs = x.stride(0), x.stride(1), out.stride(0), out.stride(1)
+        seg = tiles = None
+        max_tiles = 0
+    else:
+        seg, tiles = segments
+        _i32(seg, "seg", g + 1)
+        _i32(tiles, "tile_start", g + 1)
+        if x.dim() != 2 or out.dim() != 2 or x.stride(1) != 1 or out.stride(1) != 1:
+            raise ValueError("x and out must be matrices with unit inner stride")
+        if x.shape[1] != k or tuple(out.shape) != (x.shape[0], n_out):
+            raise ValueError(f"x {tuple(x.shape)} and out {tuple(out.shape)} do not fit w {tuple(w.shape)}")
+        m = x.shape[0]
+        x_ld, x_gs, out_ld, out_gs = x.stride(0), 0, out.stride(0), 0
+        max_tiles = -(-m // GROUPED_TILE) + g
+    z_ld = z_gs = 0
+    z = None
+    if epilogue == "gated":
+        if gate is None or gate.dtype != torch.float32 or gate.dim() != 2 or gate.stride(1) != 1 or gate.shape[0] != m:
+            raise ValueError("the gated epilogue needs float32 gate products [M, columns]")
+        if gate_column < 0 or gate_column + g * n > gate.shape[1]:
+            raise ValueError("the gate's columns lie outside the gate products")
+        z, z_ld, z_gs = gate[:, gate_column:], gate.stride(0), n
+    if m == 0:
+        return out
+    _check(load("grouped_gemm").llms_grouped_fma(
+        c_int(_code(x)), c_int(_code(out)), c_int(_EPILOGUES[epilogue]), _ptr(out), c_long(out_ld), c_long(out_gs), _ptr(x),
+        c_long(x_ld), c_long(x_gs), _ptr(w), c_int(m), c_int(n), c_int(k), c_int(g), _ptr(seg), _ptr(tiles), c_int(max_tiles),
+        _ptr(z), c_long(z_ld), c_long(z_gs), c_float(limit), _stream(dev)), "grouped_product")
+    return out
+
+
+# ------------------------------------------------------------------------------ routing to experts
+
+MOE_MAX_TOP = 16
+
+
+def moe_router(chosen: torch.Tensor, weight: torch.Tensor, h: torch.Tensor, w_router: torch.Tensor, *,
+               renormalize: bool = False) -> None:
+    """Per row of h [N, hidden]: scores sigmoid(W_router h) in 32-bit, the `top` largest in descending order (the
+    lower expert wins a tie) into chosen int32 [N, top], their scores (over their sum with `renormalize`) into
+    weight float32 [N, top]."""
+    dev = _dev(chosen, weight, h, w_router)
+    _rows(h, "h")
+    _rows(w_router, "w_router", h.shape[1])
+    n, top = h.shape[0], chosen.shape[-1]
+    _i32(chosen, "chosen", n * top)
+    _f32(weight, "weight", n * top)
+    experts = w_router.shape[0]
+    if h.dtype != w_router.dtype:
+        raise ValueError("h and w_router differ in dtype")
+    if not 1 <= top <= min(MOE_MAX_TOP, experts):
+        raise ValueError(f"1 to {MOE_MAX_TOP} choices among {experts} experts, got {top}")
+    if n == 0:
+        return
+    _check(load("moe").llms_moe_router(
+        c_int(_code(h)), _ptr(chosen), _ptr(weight), _ptr(h), _ptr(w_router), c_int(n), c_int(h.shape[1]), c_int(experts),
+        c_int(top), c_int(1 if renormalize else 0), _stream(dev)), "moe_router")
+
+
+def moe_sort(chosen: torch.Tensor, experts: int, tile: int = GROUPED_TILE):
+    """(rank [pairs], seg [E + 1], tile_start [E + 1]) of the pairs (token, choice) sorted by expert, stably: pair p's
+    row is seg[chosen[p]] + rank[p]."""
+    dev = _dev(chosen)
+    _i32(chosen, "chosen")
+    pairs = chosen.numel()
+    work = torch.empty(pairs + 3 * experts + 2, dtype=torch.int32, device=dev)
+    count, rank = work[:experts], work[experts: experts + pairs]
+    seg = work[experts + pairs: 2 * experts + pairs + 1]
+    tiles = work[2 * experts + pairs + 1:]
+    if pairs:
+        _check(load("moe").llms_moe_sort(_ptr(count), _ptr(rank), _ptr(seg), _ptr(tiles), _ptr(chosen), c_int(pairs),
+                                         c_int(experts), c_int(tile), _stream(dev)), "moe_sort")
+    return rank, seg, tiles
+
+
+def moe_scatter(xs: torch.Tensor, place: torch.Tensor, h: torch.Tensor, chosen: torch.Tensor, weight: torch.Tensor,
+                rank: torch.Tensor, seg: torch.Tensor) -> None:
+    """xs[seg[chosen[p]] + rank[p]] = weight[p] * h[p // top] (rounded to xs's dtype); place[p] = that row."""
+    dev = _dev(xs, place, h, chosen, weight, rank, seg)
+    _rows(h, "h")
+    pairs = chosen.numel()
+    _rows(xs, "xs", h.shape[1])
+    top = pairs // max(h.shape[0], 1)
+    if xs.shape[0] != pairs or xs.dtype != h.dtype or top * h.shape[0] != pairs:
+        raise ValueError("xs has a row per pair, in h's dtype")
+    _i32(place, "place", pairs)
+    _i32(chosen, "chosen", pairs)
+    _i32(rank, "rank", pairs)
+    _i32(seg, "seg")
+    _f32(weight, "weight", pairs)
+    if pairs == 0:
+        return
+    _check(load("moe").llms_moe_scatter(c_int(_code(h)), _ptr(xs), _ptr(place), _ptr(h), _ptr(chosen), _ptr(weight), _ptr(rank),
+                                        _ptr(seg), c_int(pairs), c_int(h.shape[1]), c_int(top), _stream(dev)), "moe_scatter")
+
+
+def moe_combine(y: torch.Tensor, rows: torch.Tensor, place: torch.Tensor) -> torch.Tensor:
+    """y[n] = sum_k rows[place[n, k]] in the order of k; y float32 [N, hidden], rows float32 [pairs, hidden]."""
+    dev = _dev(y, rows, place)
+    n, hidden = y.shape
+    _f32(y, "y")
+    _f32(rows, "rows")
+    _i32(place, "place", rows.shape[0])
+    top = rows.shape[0] // max(n, 1)
+    if rows.shape[1] != hidden or top * n != rows.shape[0]:
+        raise ValueError("rows has top rows of y's width per row of y")
+    if n == 0:
+        return y
+    _check(load("moe").llms_moe_combine(_ptr(y), _ptr(rows), _ptr(place), c_int(n), c_int(hidden), c_int(top), _stream(dev)),
+           "moe_combine")
+    return y

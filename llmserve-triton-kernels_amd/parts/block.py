@@ -6,6 +6,11 @@ where each g is the branch's gate (a part of the family "gate"; kind "none": no 
 stream x is 32-bit whatever the model's dtype: the branches' results arrive unrounded and one kernel
 applies the gates and sums.
 
+"streams" is the pre-norm layer over a 32-bit residual stream of one or several parallel copies:
+    x <- write_1(x, mixer(norm1(read_1(x))));  x <- write_2(x, feed_forward(norm2(read_2(x))))
+where read and write are the sublayer's `Connection` (kind "residual": read is x itself and write adds; kind "hyper":
+weighted sums over the copies).  Each write is left open and done by the kernel that reads the streams next.
+
 "prenorm" is the reference's decoder layer (src/llmserve/model/llama.py:131-135):
     x = x + mixer(norm1(x));  x = x + feed_forward(norm2(x))
 The hidden state travels as (x, delta) with the last sum still open, so each residual
@@ -18,7 +23,7 @@ import torch
 
 from ..ops import library as ops
 from .linear import linear
-from .registry import ADDED_IN_PLACE, Block, DeferredNorm, GatedSum, register_block
+from .registry import ADDED_IN_PLACE, Block, DeferredNorm, GatedSum, OpenStreams, register_block
 
 
 @register_block("prenorm")
@@ -105,3 +110,37 @@ class ParallelBlock(Block):
             return x, GatedSum(branches, z)
         ops.gated_add(x, branches, z)
         return x, None
+
+
+@register_block("streams")
+class StreamsBlock(Block):
+    """Pre-norm sublayers that meet the residual stream through connections; the stream is float32 [N, S, hidden]
+    whatever the model's dtype (the embedding's [N, hidden] becomes S equal copies at the first read).  The
+    feed-forward may be of kind "none": the layer then has a mixer only, and its second norm and connection are unused."""
+
+    ROLES = {"mixer": "mixer", "feed_forward": "feed_forward", "mixer_norm": "norm", "feed_forward_norm": "norm",
+             "mixer_connection": "connection", "feed_forward_connection": "connection"}
+
+    def _read(self, norm, connection, x, delta):
+        if not getattr(norm, "closes_streams", False):
+            raise ValueError(f"{type(norm).__name__} cannot read a stream of several copies")
+        if x.dim() == 2:  # the embedding's output: every copy starts as it
+            if delta is not None:
+                raise ValueError("an open write before the streams exist")
+            streams = torch.empty((x.shape[0], connection.streams, x.shape[1]), dtype=torch.float32, device=x.device)
+            return norm.read_streams(streams, None, connection, source=x), streams
+        if x.shape[1] != connection.streams:
+            raise ValueError(f"the stream has {x.shape[1]} copies, the connection {connection.streams}")
+        return norm.read_streams(x, delta, connection), x
+
+    def forward(self, x, delta, batch, cache):
+        h, x = self._read(self.mixer_norm, self.mixer_connection, x, delta)
+        delta = OpenStreams(self._result(self.mixer.forward(h, batch, cache)), self.mixer_connection)
+        if getattr(self.feed_forward, "absent", False):
+            return x, delta
+        h, x = self._read(self.feed_forward_norm, self.feed_forward_connection, x, delta)
+        return x, OpenStreams(self._result(self.feed_forward.forward(h)), self.feed_forward_connection)
+
+    @staticmethod
+    def _result(y):
+        return y if y.dtype == torch.float32 else y.float()

@@ -1,0 +1,81 @@
+"""A feed-forward of many small experts, of which each token uses `top`.
+
+Parameters (a `PartSpec` of kind "experts"): hidden, intermediate (of one expert), experts, top, limit,
+renormalize (default False: the weights are the chosen scores as they are), names (local names: "router", and the
+pattern of an expert's matrices, default "e{e}.gate", "e{e}.up", "e{e}.down").
+
+Router: z = W_router h in 32-bit, scores sigmoid(z), the `top` largest chosen.  The weight multiplies the expert's
+*input*: y = sum over chosen e of expert_e(w_e h).  Expert: a = min(W_gate x, limit), b = clamp(W_up x, -limit,
+limit), W_down (a sigmoid(1.702 a) (b + 1)).  No biases.
+
+One step: route, sort the (token, choice) pairs by expert on the device (stably, so a pair's place does not depend
+on what else is in the batch beyond which rows share its tile), scatter the weighted inputs into that order, two
+products with a weight per segment of rows (the first with the gated unit in its epilogue: gate and up rows
+alternate in one stacked weight), and a sum over each token's choices in their order.  Nothing is read back: the
+grids are sized by the number of pairs.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..ops import library as ops
+from .registry import FeedForward, register_feed_forward
+from .spec import ParamInfo
+
+_DEFAULT_NAMES = {"router": "router", "gate": "e{e}.gate", "up": "e{e}.up", "down": "e{e}.down"}
+
+
+@register_feed_forward("experts")
+class Experts(FeedForward):
+    graph_safe = True
+
+    def __init__(self, spec, ctx):
+        super().__init__(spec, ctx)
+        self.hidden = int(spec["hidden"])
+        self.intermediate = int(spec["intermediate"])
+        self.experts = int(spec["experts"])
+        self.top = int(spec["top"])
+        self.limit = float(spec["limit"])
+        self.renormalize = bool(spec.get("renormalize", False))
+        self.names = dict(_DEFAULT_NAMES, **(spec.get("names") or {}))
+        if not 1 <= self.top <= min(self.experts, ops.MOE_MAX_TOP):
+            raise ValueError(f"top={self.top} of {self.experts} experts (at most {ops.MOE_MAX_TOP})")
+        self.w_router = self.w_gate_up = self.w_down = None
+
+    def libraries(self, dtype_name):
+        return ("moe", "grouped_gemm")
+
+    def param_infos(self):
+        h, i, n = self.hidden, self.intermediate, self.names
+        infos = {n["router"]: ParamInfo((self.experts, h))}
+        for e in range(self.experts):
+            infos[n["gate"].format(e=e)] = ParamInfo((i, h))
+            infos[n["up"].format(e=e)] = ParamInfo((i, h))
+            infos[n["down"].format(e=e)] = ParamInfo((h, i))
+        return infos
+
+    def load(self, tensors):
+        n = self.names
+        self.w_router = tensors[n["router"]].contiguous()
+        # [E, 2 I, H] with gate and up rows alternating, so that a thread of the product holds both of a unit
+        self.w_gate_up = torch.stack([
+            torch.stack([tensors[n["gate"].format(e=e)], tensors[n["up"].format(e=e)]], dim=1).reshape(
+                2 * self.intermediate, self.hidden) for e in range(self.experts)]).contiguous()
+        self.w_down = torch.stack([tensors[n["down"].format(e=e)] for e in range(self.experts)]).contiguous()
+
+    def forward(self, x):
+        rows, dev = x.shape[0], x.device
+        pairs = rows * self.top
+        chosen = torch.empty((rows, self.top), dtype=torch.int32, device=dev)
+        weight = torch.empty((rows, self.top), dtype=torch.float32, device=dev)
+        ops.moe_router(chosen, weight, x, self.w_router, renormalize=self.renormalize)
+        rank, seg, tiles = ops.moe_sort(chosen, self.experts)
+        sorted_in = torch.empty((pairs, self.hidden), dtype=x.dtype, device=dev)
+        place = torch.empty(pairs, dtype=torch.int32, device=dev)
+        ops.moe_scatter(sorted_in, place, x, chosen, weight, rank, seg)
+        act = torch.empty((pairs, self.intermediate), dtype=x.dtype, device=dev)
+        ops.grouped_product(act, sorted_in, self.w_gate_up, epilogue="paired", segments=(seg, tiles), limit=self.limit)
+        results = torch.empty((pairs, self.hidden), dtype=torch.float32, device=dev)
+        ops.grouped_product(results, act, self.w_down, segments=(seg, tiles))
+        return ops.moe_combine(torch.empty((rows, self.hidden), dtype=torch.float32, device=dev), results, place)

@@ -11,8 +11,9 @@ from __future__ import annotations
 
 import torch
 
-from . import attention, attention_composed, block, embedding, gate, rmsnorm, rope, swiglu  # noqa: F401  (register the built-in parts)
-from .registry import BLOCKS, EMBEDDINGS, FEED_FORWARDS, GATES, HEADS, MIXERS, NORMS, BuildContext, DeferredNorm, Part
+from . import (attention, attention_composed, attention_latent, block, connection, embedding, experts, gate,  # noqa: F401
+               layernorm, rmsnorm, rope, swiglu)  # (register the built-in parts)
+from .registry import BLOCKS, CONNECTIONS, EMBEDDINGS, FEED_FORWARDS, GATES, HEADS, MIXERS, NORMS, BuildContext, DeferredNorm, Part
 from .spec import ModelSpec, ParamInfo
 
 
@@ -26,7 +27,8 @@ class Model:
         self.head = HEADS.build(spec.head, ctx)
         self.blocks = []
         self._sources = None
-        families = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS, "gate": GATES}
+        families = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS, "gate": GATES,
+                    "connection": CONNECTIONS}
         for index, layer in enumerate(spec.layers):
             block = BLOCKS.get(layer.block)
             if set(layer.parts) != set(block.ROLES) or set(layer.weights) != set(block.ROLES):

@@ -112,6 +112,16 @@ class GatedSum:
     gate_products: "torch.Tensor | None"
 
 
+@dataclass
+class OpenStreams:
+    """A write into a residual stream of several copies that is still open: new_t = sum_s mix[s, t] x_s + write[t] y,
+    with the coefficients of `connection` (a `Connection`).  It travels in the place of `delta`; a norm that sets
+    `closes_streams` does the write in the kernel that reads the streams for the next sublayer."""
+
+    y: torch.Tensor
+    connection: "Connection"
+
+
 def as_tensor(delta):
     """`delta` as a tensor in the model's dtype (None stays None)."""
     return delta.total() if isinstance(delta, PartialSums) else delta
@@ -210,11 +220,20 @@ class Gate(Part):
         return None
 
 
+class Connection(Part):
+    """How a sublayer meets a residual stream of `streams` copies [N, S, hidden]: it reads u = sum_s read[s] x_s and
+    its result y is written as new_t = sum_s mix[s, t] x_s + write[t] y.  `read`, `mix` [from, to] and `write` are
+    float32 tensors on the device, or None for the plain residual sum of one stream (u = x, x += y)."""
+
+    streams = 1
+    read = mix = write = None
+
+
 class Block:
     """Arrangement of one layer's parts.
 
     `ROLES` maps every role of the arrangement to the family its part is built from ("mixer",
-    "feed_forward", "norm" or "gate"); the model builds a part for each role from the layer's spec and hands them
+    "feed_forward", "norm", "gate" or "connection"); the model builds a part for each role from the layer's spec and hands them
     over, and they are the block's attributes by role.  The part in the role "mixer", if the arrangement
     has one, is the one that keeps a cache between steps."""
 
@@ -265,6 +284,7 @@ MIXERS = Registry("mixer")
 FEED_FORWARDS = Registry("feed-forward")
 BLOCKS = Registry("block")
 GATES = Registry("gate")
+CONNECTIONS = Registry("stream connection")
 EMBEDDINGS = Registry("embedding")
 HEADS = Registry("output head")
 
@@ -274,3 +294,4 @@ register_mixer = MIXERS.register
 register_feed_forward = FEED_FORWARDS.register
 register_block = BLOCKS.register
 register_gate = GATES.register
+register_connection = CONNECTIONS.register

@@ -73,6 +73,7 @@ class NoFeedForward(FeedForward):
     """A layer without a feed-forward: nothing joins the stream."""
 
     graph_safe = True
+    absent = True
 
     def forward(self, x):
         return None
