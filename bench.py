@@ -26,12 +26,13 @@ first token, inter-token latency percentiles and the number of preemptions besid
 `--pages-fraction` shrinks the cache pool below what the whole workload needs, so that
 requests wait and are preempted.
 
-    python bench.py --workload designs [--sizes 1b,7b] [--layers 6] [--batches 8,32] [--context 512]
+    python bench.py --workload designs [--design dibepel|milozen] [--sizes 1b,7b] [--layers 6] [--batches 8,32] [--context 512]
 
-puts the Dibepel design beside the Llama decoder at equal layer sizes (width, heads, key/value heads, head size,
+puts the Dibepel design (or, with `--design milozen`, the Milozen design: latent attention, experts, two streams)
+beside the Llama decoder at equal layer sizes (width, heads, key/value heads, head size,
 feed-forward, vocabulary, layers; random weights): prefill tokens a second for one prompt of 2,048 tokens in one
 step, and decoded tokens a second at the given batch sizes behind `--context` tokens, both through the step
-function alone (no sampling); `value` is Dibepel's decode rate at the first size and batch.
+function alone (no sampling); `value` is the design's decode rate at the first size and batch.
 """
 
 from __future__ import annotations
@@ -215,6 +216,26 @@ def dibepel_config(size: dict, layers: int, window: int = 1024, keep_first: int 
             "norm": {"eps": 1e-5}, "layers": entries}
 
 
+def milozen_config(size: dict, layers: int, window: int = 1024, experts: int = 8, top: int = 2, streams: int = 2) -> dict:
+    """As many heads as the Llama shape, each with the head size unrotated and half of it rotated, a latent of four
+    head sizes for keys and values and of three eighths of the width for queries; the first layer's feed-forward is
+    dense, the others choose `top` of `experts` experts that together are as wide as the dense one; every third layer
+    reads the cache rows of the layer before it."""
+    dim = size["dim"]
+    entries = []
+    for i in range(layers):
+        mixer = {"heads": size["heads"], "dim": dim, "rot_dim": dim // 2, "vdim": dim, "q_rank": 3 * size["width"] // 8,
+                 "kv_rank": 4 * dim, "scale": (dim + dim // 2) ** -0.5, "mask": {"size": window},
+                 "rot": {"base": 10000.0, "dims": dim // 2}}
+        if i % 3 == 2:
+            mixer["kv_from"] = i - 1
+        mlp = {"kind": "dense", "ff": size["ff"]} if i == 0 else {
+            "kind": "moe", "expert": {"ff": size["ff"] // top, "limit": 7.0}, "router": {"experts": experts, "top": top}}
+        entries.append({"type": "latent_attention", "mixer": mixer, "mlp": mlp})
+    return {"architecture": "Milozen", "vocab": size["vocab"], "width": size["width"], "embedding": {"scale": 1.0},
+            "norm": {"eps": 1e-5}, "streams": streams, "layers": entries}
+
+
 def llama_config(size: dict, layers: int, positions: int) -> dict:
     return dict(architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=size["vocab"], hidden_size=size["width"],
                 intermediate_size=size["ff"], num_hidden_layers=layers, num_attention_heads=size["heads"],
@@ -288,20 +309,23 @@ def designs(args) -> int:
         return out
 
     table = {}
+    design = args.design
+    make = {"dibepel": dibepel_config, "milozen": milozen_config}[design]
     for name in [s for s in args.sizes.split(",") if s]:
         size = DESIGN_SIZES[name]
         layers = args.layers or 6
-        row = {"layers": layers, **size, "dibepel": measure(dibepel_config(size, layers)),
+        row = {"layers": layers, **size, design: measure(make(size, layers)),
                "llama": measure(llama_config(size, layers, longest))}
-        row["dibepel_over_llama"] = {k: round(row["dibepel"][k] / row["llama"][k], 3) for k in row["dibepel"]
-                                     if k.endswith("tok_s")}
+        row[f"{design}_over_llama"] = {k: round(row[design][k] / row["llama"][k], 3) for k in row[design]
+                                       if k.endswith("tok_s")}
         table[name] = row
     first = table[next(iter(table))]
-    line = {"metric": "Dibepel beside Llama at equal layer sizes: decode tok/s (value: Dibepel, first size and batch), prefill tok/s",
-            "value": first["dibepel"][f"decode_b{batches[0]}_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": steps,
-            "warmup": warmup, "ms_per_step": first["dibepel"][f"decode_b{batches[0]}_ms"], "higher_is_better": True,
+    title = design.capitalize()
+    line = {"metric": f"{title} beside Llama at equal layer sizes: decode tok/s (value: {title}, first size and batch), prefill tok/s",
+            "value": first[design][f"decode_b{batches[0]}_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": steps,
+            "warmup": warmup, "ms_per_step": first[design][f"decode_b{batches[0]}_ms"], "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
-            "data": "synthetic", "config": {"model": "dibepel at llama layer sizes", "global_batch": batches[0],
+            "data": "synthetic", "config": {"model": f"{design} at llama layer sizes", "global_batch": batches[0],
                                             "seq_len": args.context, "parallelism": "single-gpu", "weights": "random",
                                             "prefill_tokens": PREFILL_TOKENS},
             "designs": table}
@@ -428,6 +452,7 @@ def main() -> int:
                     help="run one phase only (for profiles; the line then holds zeros for the other); gemv: the "
                          "decode products alone, each over copies of its weight that do not fit the caches")
     ap.add_argument("--workload", choices=["steps", "serve", "designs"], default="steps")
+    ap.add_argument("--design", choices=["dibepel", "milozen"], default="dibepel", help="designs: which design stands beside Llama")
     ap.add_argument("--sizes", default="1b,7b", help="designs: layer sizes to compare at")
     ap.add_argument("--batches", default="8,32", help="designs: decode batch sizes")
     ap.add_argument("--requests", type=int, default=64)

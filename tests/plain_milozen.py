@@ -165,3 +165,10 @@ def forward(config: dict, tensors: dict, tokens, dtype=torch.float64, layers_out
             layers_out.append(xs.sum(dim=0).clone())
     x = xs.sum(dim=0)
     return layer_norm(x, ts["final.norm"], eps) @ ts["embed"].T
+
+
+def greedy(config: dict, tensors: dict, prompt, n_new: int, dtype=torch.float64) -> list[int]:
+    ids = list(prompt)
+    for _ in range(n_new):
+        ids.append(int(forward(config, tensors, ids, dtype)[-1].argmax()))
+    return ids[len(prompt):]
