@@ -3,10 +3,12 @@
 //                             the columns g * out_gs .. of out (a product per head)
 //   groups as row segments    rows seg[g] .. seg[g + 1] belong to group g (rows sorted by expert); a workgroup finds
 //                             its group and tile from tile_start[g] = tiles of all groups before g
-// Epilogues: plain; "paired" for a weight whose rows alternate between two projections a, b of a gated unit:
-// out[m, n / 2] = min(a, limit) * sigmoid(1.702 min(a, limit)) * (clamp(b, -limit, limit) + 1); "gated": the result
-// times sigmoid(z[m, g * z_gs + n]) with z in 32-bit.
-// This file holds the 32-bit multiply-add kernel (any sizes, float or bfloat16 operands, 32-bit products and sums).
+// Epilogues: plain; "paired" for a weight that stacks two projections a, b of a gated unit in blocks of 64 rows (32
+// rows of a, then the 32 rows of b of the same units, so that a thread or lane holds both of a unit):
+// out[m, u] = min(a, limit) * sigmoid(1.702 min(a, limit)) * (clamp(b, -limit, limit) + 1) for the `units` units;
+// "gated": the result times sigmoid(z[m, g * z_gs + n]) with z in 32-bit.
+// Two kernels: 32-bit multiply-add (any sizes, float or bfloat16 operands, 32-bit products and sums) and bfloat16 on
+// the matrix cores (K and the strides of x in multiples of 8, 16-byte aligned operands).
 #include "common.h"
 
 #define GG_TM 64
@@ -17,11 +19,19 @@
 #define GG_PAIRED 1
 #define GG_GATED 2
 
+// (the operands of the gated unit are rounded as a stored activation would be)
+template <typename TOut>
+__device__ __forceinline__ float gated_unit(float a_sum, float b_sum, float limit) {
+    const float a = fminf(round_to<TOut>(a_sum), limit);
+    const float b = fminf(fmaxf(round_to<TOut>(b_sum), -limit), limit);
+    return a / (1.f + expf(-1.702f * a)) * (b + 1.f);
+}
+
 template <typename TIn, typename TOut, int EPI>
 __global__ __launch_bounds__(256) void grouped_fma_kernel(
     TOut* __restrict__ out, long out_ld, long out_gs, const TIn* __restrict__ x, long x_ld, long x_gs,
     const TIn* __restrict__ w, int M, int N, int K, int G, const int* __restrict__ seg, const int* __restrict__ tile_start,
-    const float* __restrict__ z, long z_ld, long z_gs, float limit) {
+    const float* __restrict__ z, long z_ld, long z_gs, float limit, int units) {
     __shared__ float As[GG_TK][GG_TM + 4];
     __shared__ float Ws[GG_TK][GG_TN + 4];
     const int tid = threadIdx.x;
@@ -41,7 +51,9 @@ __global__ __launch_bounds__(256) void grouped_fma_kernel(
     const int n0 = blockIdx.x * GG_TN;
     const TIn* xg = x + (seg ? 0 : (size_t)g * x_gs);
     const TIn* wg = w + (size_t)g * N * K;
-    const int tm = (tid / 16) * 4, tn = (tid % 16) * 4;
+    // a thread's four columns: two neighbours in the first half of the tile and the same two in the second half
+    const int tm = (tid / 16) * 4, tn = (tid % 16) * 2;
+    auto column = [&](int j) { return tn + (j & 1) + 32 * (j >> 1); };
     const int lr = tid / 4, lk = (tid % 4) * 4;
     float acc[4][4] = {};
     for (int k0 = 0; k0 < K; k0 += GG_TK) {
@@ -59,7 +71,7 @@ __global__ __launch_bounds__(256) void grouped_fma_kernel(
 #pragma unroll
             for (int i = 0; i < 4; ++i) a[i] = As[k][tm + i];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) b[j] = Ws[k][tn + j];
+            for (int j = 0; j < 4; ++j) b[j] = Ws[k][column(j)];
 #pragma unroll
             for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -74,18 +86,15 @@ __global__ __launch_bounds__(256) void grouped_fma_kernel(
         if (m >= row_end) continue;
         if (EPI == GG_PAIRED) {
 #pragma unroll
-            for (int j = 0; j < 4; j += 2) {
-                const int n = n0 + tn + j;
-                if (n + 1 >= N) continue;
-                // (the operands of the second product are rounded as a stored activation would be)
-                const float a = fminf(round_to<TOut>(acc[i][j]), limit);
-                const float b = fminf(fmaxf(round_to<TOut>(acc[i][j + 1]), -limit), limit);
-                og[(size_t)m * out_ld + n / 2] = from_f32<TOut>(a / (1.f + expf(-1.702f * a)) * (b + 1.f));
+            for (int j = 0; j < 2; ++j) {
+                const int u = n0 / 2 + tn + j;
+                if (u >= units) continue;
+                og[(size_t)m * out_ld + u] = from_f32<TOut>(gated_unit<TOut>(acc[i][j], acc[i][j + 2], limit));
             }
         } else {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const int n = n0 + tn + j;
+                const int n = n0 + column(j);
                 if (n >= N) continue;
                 float v = acc[i][j];
                 if (EPI == GG_GATED) v = v / (1.f + expf(-z[(size_t)m * z_ld + (size_t)g * z_gs + n]));
@@ -98,14 +107,144 @@ __global__ __launch_bounds__(256) void grouped_fma_kernel(
 template <typename TIn, typename TOut>
 static int launch_fma(int epilogue, dim3 grid, hipStream_t stream, void* out, long out_ld, long out_gs, const void* x, long x_ld,
                       long x_gs, const void* w, int M, int N, int K, int G, const int* seg, const int* tile_start, const float* z,
-                      long z_ld, long z_gs, float limit) {
+                      long z_ld, long z_gs, float limit, int units) {
 #define GG_GO(EPI)                                                                                                          \
     grouped_fma_kernel<TIn, TOut, EPI><<<grid, 256, 0, stream>>>((TOut*)out, out_ld, out_gs, (const TIn*)x, x_ld, x_gs,      \
-                                                                 (const TIn*)w, M, N, K, G, seg, tile_start, z, z_ld, z_gs, limit)
+                                                                 (const TIn*)w, M, N, K, G, seg, tile_start, z, z_ld, z_gs, limit, units)
     if (epilogue == GG_PLAIN) GG_GO(GG_PLAIN);
     else if (epilogue == GG_PAIRED) GG_GO(GG_PAIRED);
     else GG_GO(GG_GATED);
 #undef GG_GO
+    LLMS_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------------------ bfloat16 on the matrix cores
+// 128 x 128 tiles through double-buffered LDS, 4 waves of 64 x 64, v_mfma_f32_32x32x16_bf16: lane l holds
+// A[i = l%32][k = 8*(l/32) .. +7] and B[k = same][j = l%32]; result D[i = 8*(r/4) + 4*(l/32) + r%4][j = l%32].
+// Here i = row m and j = weight row n, so a wave's two column blocks of 32 are the a and b rows of the same 32 units
+// of a paired weight (columns 0..31 and 32..63 of its 64), both in the same lane.
+typedef __attribute__((ext_vector_type(8))) __bf16 gg_bf16x8;
+typedef __attribute__((ext_vector_type(16))) float gg_f32x16;
+typedef __attribute__((ext_vector_type(4))) uint32_t gg_u32x4;
+
+#define GM_BM 128
+#define GM_BN 128
+#define GM_BK 32
+#define GM_LD 40  // LDS row stride in elements: 32 + 8 of padding against bank conflicts
+
+template <typename TOut, int EPI>
+__global__ __launch_bounds__(256) void grouped_mfma_kernel(
+    TOut* __restrict__ out, long out_ld, long out_gs, const bf16* __restrict__ x, long x_ld, long x_gs,
+    const bf16* __restrict__ w, int M, int N, int K, int G, const int* __restrict__ seg, const int* __restrict__ tile_start,
+    const float* __restrict__ z, long z_ld, long z_gs, float limit, int units) {
+    __shared__ __attribute__((aligned(16))) uint16_t As[2][GM_BM * GM_LD];
+    __shared__ __attribute__((aligned(16))) uint16_t Bs[2][GM_BN * GM_LD];
+    int g, row0, row_end;
+    if (seg) {
+        const int t = blockIdx.y;
+        if (t >= tile_start[G]) return;
+        g = 0;
+        while (tile_start[g + 1] <= t) ++g;  // (uniform over the workgroup)
+        row0 = seg[g] + (t - tile_start[g]) * GM_BM;
+        row_end = seg[g + 1];
+    } else {
+        g = blockIdx.z;
+        row0 = blockIdx.y * GM_BM;
+        row_end = M;
+    }
+    const int n0 = blockIdx.x * GM_BN;
+    const bf16* xg = x + (seg ? 0 : (size_t)g * x_gs);
+    const bf16* wg = w + (size_t)g * N * K;
+    const int tid = threadIdx.x, wave = tid / LLMS_WAVE, lane = tid % LLMS_WAVE;
+    const int wm = (wave % 2) * 64, wn = (wave / 2) * 64;
+    const int l32 = lane % 32, hi = lane / 32;
+    const gg_u32x4 zero = {0, 0, 0, 0};
+    gg_f32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    // staging: 512 pieces of 8 elements per operand tile, two per thread
+    gg_u32x4 ra[2], rb[2];
+    const int crow[2] = {tid / 4, (tid + 256) / 4};
+    const int ckc = (tid % 4) * 8;
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            const int k = k0 + ckc;
+            const int am = row0 + crow[c], wr = n0 + crow[c];
+            ra[c] = (am < row_end && k < K) ? *reinterpret_cast<const gg_u32x4*>(xg + (size_t)am * x_ld + k) : zero;
+            rb[c] = (wr < N && k < K) ? *reinterpret_cast<const gg_u32x4*>(wg + (size_t)wr * K + k) : zero;
+        }
+    };
+    auto stage = [&](int buf) {
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            *reinterpret_cast<gg_u32x4*>(&As[buf][crow[c] * GM_LD + ckc]) = ra[c];
+            *reinterpret_cast<gg_u32x4*>(&Bs[buf][crow[c] * GM_LD + ckc]) = rb[c];
+        }
+    };
+    const int ktiles = (K + GM_BK - 1) / GM_BK;
+    fetch(0);
+    stage(0);
+    __syncthreads();
+    for (int kt = 0; kt < ktiles; ++kt) {
+        const int buf = kt & 1;
+        if (kt + 1 < ktiles) fetch((kt + 1) * GM_BK);
+#pragma unroll
+        for (int s = 0; s < GM_BK / 16; ++s) {
+            gg_bf16x8 af[2], bfr[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                af[i] = __builtin_bit_cast(gg_bf16x8, *reinterpret_cast<const gg_u32x4*>(&As[buf][(wm + i * 32 + l32) * GM_LD + s * 16 + hi * 8]));
+                bfr[i] = __builtin_bit_cast(gg_bf16x8, *reinterpret_cast<const gg_u32x4*>(&Bs[buf][(wn + i * 32 + l32) * GM_LD + s * 16 + hi * 8]));
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+        }
+        if (kt + 1 < ktiles) stage(buf ^ 1);
+        __syncthreads();
+    }
+    TOut* og = out + (seg ? 0 : (size_t)g * out_gs);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int m = row0 + wm + i * 32 + 8 * (r / 4) + 4 * hi + (r % 4);
+            if (m >= row_end) continue;
+            if (EPI == GG_PAIRED) {
+                const int u = (n0 + wn) / 2 + l32;
+                if (u < units) og[(size_t)m * out_ld + u] = from_f32<TOut>(gated_unit<TOut>(acc[i][0][r], acc[i][1][r], limit));
+            } else {
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int n = n0 + wn + j * 32 + l32;
+                    if (n >= N) continue;
+                    float v = acc[i][j][r];
+                    if (EPI == GG_GATED) v = v / (1.f + expf(-z[(size_t)m * z_ld + (size_t)g * z_gs + n]));
+                    og[(size_t)m * out_ld + n] = from_f32<TOut>(v);
+                }
+            }
+        }
+    }
+}
+
+template <typename TOut>
+static int launch_mfma(int epilogue, dim3 grid, hipStream_t stream, void* out, long out_ld, long out_gs, const void* x, long x_ld,
+                       long x_gs, const void* w, int M, int N, int K, int G, const int* seg, const int* tile_start, const float* z,
+                       long z_ld, long z_gs, float limit, int units) {
+#define GM_GO(EPI)                                                                                                          \
+    grouped_mfma_kernel<TOut, EPI><<<grid, 256, 0, stream>>>((TOut*)out, out_ld, out_gs, (const bf16*)x, x_ld, x_gs,         \
+                                                             (const bf16*)w, M, N, K, G, seg, tile_start, z, z_ld, z_gs, limit, units)
+    if (epilogue == GG_PLAIN) GM_GO(GG_PLAIN);
+    else if (epilogue == GG_PAIRED) GM_GO(GG_PAIRED);
+    else GM_GO(GG_GATED);
+#undef GM_GO
     LLMS_LAUNCH_CHECK();
 }
 
@@ -116,24 +255,48 @@ extern "C" {
 // tile_start[G], which the host bounds by ceil(M / 64) + G).
 int llms_grouped_fma(int in_dtype, int out_dtype, int epilogue, void* out, long out_ld, long out_gs, const void* x, long x_ld,
                      long x_gs, const void* w, int M, int N, int K, int G, const int* seg, const int* tile_start,
-                     int max_tiles, const float* z, long z_ld, long z_gs, float limit, hipStream_t stream) {
+                     int max_tiles, const float* z, long z_ld, long z_gs, float limit, int units, hipStream_t stream) {
     LLMS_REQUIRE(M > 0 && N > 0 && K > 0 && G > 0, "grouped_fma: sizes must be positive");
     LLMS_REQUIRE(epilogue >= 0 && epilogue <= 2, "grouped_fma: epilogue 0 (plain), 1 (paired) or 2 (gated)");
-    LLMS_REQUIRE(epilogue != GG_PAIRED || N % 2 == 0, "grouped_fma: a paired weight has an even number of rows");
+    LLMS_REQUIRE(epilogue != GG_PAIRED || (N % 64 == 0 && units > 0 && units <= N / 2),
+                 "grouped_fma: a paired weight has blocks of 64 rows for 32 units each");
     LLMS_REQUIRE(epilogue != GG_GATED || z, "grouped_fma: the gated epilogue needs its gate products");
     LLMS_REQUIRE((seg == nullptr) == (tile_start == nullptr), "grouped_fma: segments come with their tile starts");
     dim3 grid((N + GG_TN - 1) / GG_TN, seg ? max_tiles : (M + GG_TM - 1) / GG_TM, seg ? 1 : G);
     LLMS_REQUIRE(grid.y > 0 && grid.y <= 65535 && grid.z <= 65535, "grouped_fma: too many rows or groups for one launch");
     if (in_dtype == 0 && out_dtype == 0)
         return launch_fma<float, float>(epilogue, grid, stream, out, out_ld, out_gs, x, x_ld, x_gs, w, M, N, K, G, seg, tile_start,
-                                        z, z_ld, z_gs, limit);
+                                        z, z_ld, z_gs, limit, units);
     if (in_dtype == 1 && out_dtype == 1)
         return launch_fma<bf16, bf16>(epilogue, grid, stream, out, out_ld, out_gs, x, x_ld, x_gs, w, M, N, K, G, seg, tile_start, z,
-                                      z_ld, z_gs, limit);
+                                      z_ld, z_gs, limit, units);
     if (in_dtype == 1 && out_dtype == 0)
         return launch_fma<bf16, float>(epilogue, grid, stream, out, out_ld, out_gs, x, x_ld, x_gs, w, M, N, K, G, seg, tile_start, z,
-                                       z_ld, z_gs, limit);
+                                       z_ld, z_gs, limit, units);
     LLMS_REQUIRE(false, "grouped_fma: unsupported dtype pair");
+}
+
+// The same on the matrix cores: bfloat16 operands, out_dtype 0 (float32) or 1 (bfloat16); tiles of 128 rows.
+int llms_grouped_mfma(int out_dtype, int epilogue, void* out, long out_ld, long out_gs, const void* x, long x_ld, long x_gs,
+                      const void* w, int M, int N, int K, int G, const int* seg, const int* tile_start, int max_tiles,
+                      const float* z, long z_ld, long z_gs, float limit, int units, hipStream_t stream) {
+    LLMS_REQUIRE(M > 0 && N > 0 && K > 0 && G > 0, "grouped_mfma: sizes must be positive");
+    LLMS_REQUIRE(epilogue >= 0 && epilogue <= 2, "grouped_mfma: epilogue 0 (plain), 1 (paired) or 2 (gated)");
+    LLMS_REQUIRE(epilogue != GG_PAIRED || (N % 64 == 0 && units > 0 && units <= N / 2),
+                 "grouped_mfma: a paired weight has blocks of 64 rows for 32 units each");
+    LLMS_REQUIRE(epilogue != GG_GATED || z, "grouped_mfma: the gated epilogue needs its gate products");
+    LLMS_REQUIRE((seg == nullptr) == (tile_start == nullptr), "grouped_mfma: segments come with their tile starts");
+    LLMS_REQUIRE(K % 8 == 0 && x_ld % 8 == 0 && x_gs % 8 == 0, "grouped_mfma: K and the strides of x in multiples of 8");
+    LLMS_REQUIRE(((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0, "grouped_mfma: x and w must be 16-byte aligned");
+    dim3 grid((N + GM_BN - 1) / GM_BN, seg ? max_tiles : (M + GM_BM - 1) / GM_BM, seg ? 1 : G);
+    LLMS_REQUIRE(grid.y > 0 && grid.y <= 65535 && grid.z <= 65535, "grouped_mfma: too many rows or groups for one launch");
+    if (out_dtype == 0)
+        return launch_mfma<float>(epilogue, grid, stream, out, out_ld, out_gs, x, x_ld, x_gs, w, M, N, K, G, seg, tile_start, z, z_ld,
+                                  z_gs, limit, units);
+    if (out_dtype == 1)
+        return launch_mfma<bf16>(epilogue, grid, stream, out, out_ld, out_gs, x, x_ld, x_gs, w, M, N, K, G, seg, tile_start, z, z_ld,
+                                 z_gs, limit, units);
+    LLMS_REQUIRE(false, "grouped_mfma: out_dtype must be 0 or 1");
 }
 
 }  // extern "C"

@@ -1,10 +1,9 @@
 // Routing for a feed-forward of many small experts, of which each token uses `top`.
-//   moe_router    z = W_router h in 32-bit, s = sigmoid(z) (or softmax is not offered: the scores are independent),
-//                 the `top` largest (the lower expert wins a tie), in descending order; weight = score or
+//   moe_router    z = W_router h in 32-bit, s = sigmoid(z), the `top` largest (the lower expert wins a tie), in descending order; weight = score or
 //                 score / sum of the chosen scores
 //   moe_rank      for expert e: how many (token, choice) pairs chose it, and each such pair's rank among them in the
 //                 order of the pairs (so the sorted order is stable and the same whatever runs beside it)
-//   moe_offsets   seg[e] = pairs of all experts before e, tile_start[e] = tiles of `tile` rows of all experts before e
+//   moe_offsets   seg[e] = pairs of all experts before e, tile_start[e] = tiles of rows of all experts before e
 //   moe_scatter   rows sorted by expert: xs[seg[e] + rank] = weight * h[token] (the weight multiplies the expert's
 //                 input), rounded to T; place[pair] = that row
 //   moe_combine   y[n] = sum over the token's choices, in their order, of the experts' results rows (32-bit)
@@ -92,19 +91,23 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_rank_kernel(int* __restrict__
     if (threadIdx.x == 0) count[e] = base;
 }
 
-// one workgroup of one thread's work: experts are few
+// one workgroup of one thread's work: experts are few.  tile_start [2, experts + 1]: for tiles of `tile_a` and of
+// `tile_b` rows (the two kernels that multiply segments of rows have tiles of different heights)
 __global__ void moe_offsets_kernel(int* __restrict__ seg, int* __restrict__ tile_start, const int* __restrict__ count,
-                                   int experts, int tile) {
+                                   int experts, int tile_a, int tile_b) {
     if (threadIdx.x != 0 || blockIdx.x != 0) return;
-    int rows = 0, tiles = 0;
+    int rows = 0, tiles_a = 0, tiles_b = 0;
     for (int e = 0; e < experts; ++e) {
         seg[e] = rows;
-        tile_start[e] = tiles;
+        tile_start[e] = tiles_a;
+        tile_start[experts + 1 + e] = tiles_b;
         rows += count[e];
-        tiles += (count[e] + tile - 1) / tile;
+        tiles_a += (count[e] + tile_a - 1) / tile_a;
+        tiles_b += (count[e] + tile_b - 1) / tile_b;
     }
     seg[experts] = rows;
-    tile_start[experts] = tiles;
+    tile_start[experts] = tiles_a;
+    tile_start[2 * experts + 1] = tiles_b;
 }
 
 // grid: pairs
@@ -150,12 +153,12 @@ int llms_moe_router(int dtype, int* chosen, float* weight, const void* h, const 
     LLMS_LAUNCH_CHECK();
 }
 
-// count [E], rank [pairs], seg [E + 1], tile_start [E + 1]
-int llms_moe_sort(int* count, int* rank, int* seg, int* tile_start, const int* chosen, int pairs, int experts, int tile,
-                  hipStream_t stream) {
-    LLMS_REQUIRE(pairs > 0 && experts > 0 && tile > 0, "moe_sort: sizes must be positive");
+// count [E], rank [pairs], seg [E + 1], tile_start [2, E + 1]
+int llms_moe_sort(int* count, int* rank, int* seg, int* tile_start, const int* chosen, int pairs, int experts, int tile_a,
+                  int tile_b, hipStream_t stream) {
+    LLMS_REQUIRE(pairs > 0 && experts > 0 && tile_a > 0 && tile_b > 0, "moe_sort: sizes must be positive");
     moe_rank_kernel<<<experts, MOE_THREADS, 0, stream>>>(count, rank, chosen, pairs);
-    moe_offsets_kernel<<<1, 64, 0, stream>>>(seg, tile_start, count, experts, tile);
+    moe_offsets_kernel<<<1, 64, 0, stream>>>(seg, tile_start, count, experts, tile_a, tile_b);
     LLMS_LAUNCH_CHECK();
 }
 

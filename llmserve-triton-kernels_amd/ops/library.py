@@ -1287,27 +1287,53 @@ def attend_latent(out: torch.Tensor, q: torch.Tensor, pool: torch.Tensor, block_
 # ------------------------------------------------------------------------------ products with a weight per group
 
 c_long = ctypes.c_long
-GROUPED_TILE = 64
+GROUPED_TILE = 64  # rows of a tile of the multiply-add kernel
+GROUPED_TILE_MFMA = 128  # and of the matrix-core kernel
+PAIRED_BLOCK = 32  # units per block of a paired weight: 32 rows of the first projection, then 32 of the second
 _EPILOGUES = {"plain": 0, "paired": 1, "gated": 2}
+GROUPED_KERNEL = os.environ.get("LLMSERVE_GROUPED_GEMM", "")  # "fma": keep the matrix-core kernel out
+
+
+def stack_paired(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """[.., units, K] twice -> [.., 64 * ceil(units / 32), K]: blocks of 32 rows of a followed by the 32 rows of b of
+    the same units (rows of units that do not exist are zero): the weight of the "paired" epilogue."""
+    units, k = a.shape[-2:]
+    blocks = -(-units // PAIRED_BLOCK)
+    pad = blocks * PAIRED_BLOCK - units
+    if pad:
+        zeros = torch.zeros((*a.shape[:-2], pad, k), dtype=a.dtype, device=a.device)
+        a, b = torch.cat([a, zeros], dim=-2), torch.cat([b, zeros], dim=-2)
+    a = a.reshape(*a.shape[:-2], blocks, PAIRED_BLOCK, k)
+    b = b.reshape(*b.shape[:-2], blocks, PAIRED_BLOCK, k)
+    return torch.cat([a, b], dim=-2).reshape(*a.shape[:-3], blocks * 2 * PAIRED_BLOCK, k).contiguous()
+
+
+def _grouped_on_matrix_cores(x: torch.Tensor, w: torch.Tensor, x_ld: int, x_gs: int) -> bool:
+    return (GROUPED_KERNEL != "fma" and x.dtype == torch.bfloat16 and w.shape[2] % 8 == 0 and x_ld % 8 == 0
+            and x_gs % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
 def grouped_product(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, *, epilogue: str = "plain",
                     segments: "tuple[torch.Tensor, torch.Tensor] | None" = None, gate: torch.Tensor | None = None,
-                    gate_column: int = 0, limit: float = 0.0) -> torch.Tensor:
+                    gate_column: int = 0, limit: float = 0.0, units: int = 0) -> torch.Tensor:
     """w [G, N, K].  Without `segments` every row meets every group: x [M, G, K] and out [M, G, N'] (views whose
     last axis has unit stride; the strides of the other two are free), out[m, g] = x[m, g] w[g]^T.  With `segments`
-    = (seg [G + 1], tile_start [G + 1]) on the device, x [M, K] and out [M, N'] hold rows sorted by group, rows
-    seg[g] .. seg[g + 1] belonging to group g, and tile_start counts tiles of GROUPED_TILE rows.
-    Epilogues: "plain" (N' = N); "paired" (N' = N / 2: the weight's rows alternate between the two projections a, b of
-    a gated unit, out = min(a, limit) sigmoid(1.702 min(a, limit)) (clamp(b, +-limit) + 1)); "gated" (out times
-    sigmoid(gate[m, gate_column + g N + n]), gate float32 [M, columns])."""
+    = (seg [G + 1], tile_start [2, G + 1]) on the device (what `moe_sort` returns), x [M, K] and out [M, N'] hold rows
+    sorted by group, rows seg[g] .. seg[g + 1] belonging to group g.
+    Epilogues: "plain" (N' = N); "paired" (N' = `units`: w is `stack_paired(a, b)`,
+    out = min(a, limit) sigmoid(1.702 min(a, limit)) (clamp(b, +-limit) + 1)); "gated" (out times
+    sigmoid(gate[m, gate_column + g N + n]), gate float32 [M, columns]).
+    bfloat16 operands with K and the strides of x in multiples of 8 go to the matrix cores, all else to the 32-bit
+    multiply-add kernel."""
     dev = _dev(out, x, w, gate, *(segments or ()))
     if w.dim() != 3 or not w.is_contiguous():
         raise ValueError("w must be a contiguous [G, N, K] tensor")
     g, n, k = w.shape
-    n_out = n // 2 if epilogue == "paired" else n
-    if epilogue not in _EPILOGUES or (epilogue == "paired" and n % 2):
-        raise ValueError(f"epilogue {epilogue!r} with {n} weight rows")
+    if epilogue not in _EPILOGUES:
+        raise ValueError(f"epilogue {epilogue!r}")
+    if epilogue == "paired" and (n % (2 * PAIRED_BLOCK) or not 0 < units <= n // 2):
+        raise ValueError(f"a paired weight of {n} rows does not hold {units} units")
+    n_out = units if epilogue == "paired" else n
     if x.dtype != w.dtype or (x.dtype, out.dtype) not in ((torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
                                                          (torch.bfloat16, torch.float32)):
         raise ValueError(f"grouped_product does not take {x.dtype} x {w.dtype} -> {out.dtype}")
@@ -1318,19 +1344,23 @@ def grouped_product(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, *, epil
             raise ValueError(f"x {tuple(x.shape)} and out {tuple(out.shape)} do not fit w {tuple(w.shape)}")
         m = x.shape[0]
         x_ld, x_gs, out_ld, out_gs = x.stride(0), x.stride(1), out.stride(0), out.stride(1)
-        seg = tiles = None
-        max_tiles = 0
     else:
         seg, tiles = segments
         _i32(seg, "seg", g + 1)
-        _i32(tiles, "tile_start", g + 1)
+        _i32(tiles, "tile_start", 2 * (g + 1))
         if x.dim() != 2 or out.dim() != 2 or x.stride(1) != 1 or out.stride(1) != 1:
             raise ValueError("x and out must be matrices with unit inner stride")
         if x.shape[1] != k or tuple(out.shape) != (x.shape[0], n_out):
             raise ValueError(f"x {tuple(x.shape)} and out {tuple(out.shape)} do not fit w {tuple(w.shape)}")
         m = x.shape[0]
         x_ld, x_gs, out_ld, out_gs = x.stride(0), 0, out.stride(0), 0
-        max_tiles = -(-m // GROUPED_TILE) + g
+    mfma = _grouped_on_matrix_cores(x, w, x_ld, x_gs)
+    seg_ptr = tiles_ptr = None
+    max_tiles = 0
+    if segments is not None:
+        tile = GROUPED_TILE_MFMA if mfma else GROUPED_TILE
+        seg_ptr, tiles_ptr = seg, tiles.view(2, g + 1)[1 if mfma else 0]
+        max_tiles = -(-m // tile) + g
     z_ld = z_gs = 0
     z = None
     if epilogue == "gated":
@@ -1341,10 +1371,14 @@ def grouped_product(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, *, epil
         z, z_ld, z_gs = gate[:, gate_column:], gate.stride(0), n
     if m == 0:
         return out
-    _check(load("grouped_gemm").llms_grouped_fma(
-        c_int(_code(x)), c_int(_code(out)), c_int(_EPILOGUES[epilogue]), _ptr(out), c_long(out_ld), c_long(out_gs), _ptr(x),
-        c_long(x_ld), c_long(x_gs), _ptr(w), c_int(m), c_int(n), c_int(k), c_int(g), _ptr(seg), _ptr(tiles), c_int(max_tiles),
-        _ptr(z), c_long(z_ld), c_long(z_gs), c_float(limit), _stream(dev)), "grouped_product")
+    common = (_ptr(out), c_long(out_ld), c_long(out_gs), _ptr(x), c_long(x_ld), c_long(x_gs), _ptr(w), c_int(m), c_int(n),
+              c_int(k), c_int(g), _ptr(seg_ptr), _ptr(tiles_ptr), c_int(max_tiles), _ptr(z), c_long(z_ld), c_long(z_gs),
+              c_float(limit), c_int(units), _stream(dev))
+    lib = load("grouped_gemm")
+    if mfma:
+        _check(lib.llms_grouped_mfma(c_int(_code(out)), c_int(_EPILOGUES[epilogue]), *common), "grouped_product")
+    else:
+        _check(lib.llms_grouped_fma(c_int(_code(x)), c_int(_code(out)), c_int(_EPILOGUES[epilogue]), *common), "grouped_product")
     return out
 
 
@@ -1376,19 +1410,20 @@ def moe_router(chosen: torch.Tensor, weight: torch.Tensor, h: torch.Tensor, w_ro
         c_int(top), c_int(1 if renormalize else 0), _stream(dev)), "moe_router")
 
 
-def moe_sort(chosen: torch.Tensor, experts: int, tile: int = GROUPED_TILE):
-    """(rank [pairs], seg [E + 1], tile_start [E + 1]) of the pairs (token, choice) sorted by expert, stably: pair p's
-    row is seg[chosen[p]] + rank[p]."""
+def moe_sort(chosen: torch.Tensor, experts: int):
+    """(rank [pairs], seg [E + 1], tile_start [2, E + 1]) of the pairs (token, choice) sorted by expert, stably: pair
+    p's row is seg[chosen[p]] + rank[p]; tile_start counts the tiles of rows of all experts before each, once for the
+    tiles of the multiply-add kernel and once for those of the matrix-core kernel."""
     dev = _dev(chosen)
     _i32(chosen, "chosen")
     pairs = chosen.numel()
-    work = torch.empty(pairs + 3 * experts + 2, dtype=torch.int32, device=dev)
+    work = torch.empty(pairs + 4 * experts + 3, dtype=torch.int32, device=dev)
     count, rank = work[:experts], work[experts: experts + pairs]
     seg = work[experts + pairs: 2 * experts + pairs + 1]
     tiles = work[2 * experts + pairs + 1:]
     if pairs:
         _check(load("moe").llms_moe_sort(_ptr(count), _ptr(rank), _ptr(seg), _ptr(tiles), _ptr(chosen), c_int(pairs),
-                                         c_int(experts), c_int(tile), _stream(dev)), "moe_sort")
+                                         c_int(experts), c_int(GROUPED_TILE), c_int(GROUPED_TILE_MFMA), _stream(dev)), "moe_sort")
     return rank, seg, tiles
 
 

@@ -11,7 +11,7 @@ limit), W_down (a sigmoid(1.702 a) (b + 1)).  No biases.
 One step: route, sort the (token, choice) pairs by expert on the device (stably, so a pair's place does not depend
 on what else is in the batch beyond which rows share its tile), scatter the weighted inputs into that order, two
 products with a weight per segment of rows (the first with the gated unit in its epilogue: gate and up rows
-alternate in one stacked weight), and a sum over each token's choices in their order.  Nothing is read back: the
+lie in blocks of 32 in one stacked weight), and a sum over each token's choices in their order.  Nothing is read back: the
 grids are sized by the number of pairs.
 """
 
@@ -58,10 +58,10 @@ class Experts(FeedForward):
     def load(self, tensors):
         n = self.names
         self.w_router = tensors[n["router"]].contiguous()
-        # [E, 2 I, H] with gate and up rows alternating, so that a thread of the product holds both of a unit
-        self.w_gate_up = torch.stack([
-            torch.stack([tensors[n["gate"].format(e=e)], tensors[n["up"].format(e=e)]], dim=1).reshape(
-                2 * self.intermediate, self.hidden) for e in range(self.experts)]).contiguous()
+        # [E, 64 ceil(I / 32), H]: blocks of 32 gate rows and the 32 up rows of the same units, so that a thread of
+        # the product holds both of a unit
+        self.w_gate_up = ops.stack_paired(torch.stack([tensors[n["gate"].format(e=e)] for e in range(self.experts)]),
+                                          torch.stack([tensors[n["up"].format(e=e)] for e in range(self.experts)]))
         self.w_down = torch.stack([tensors[n["down"].format(e=e)] for e in range(self.experts)]).contiguous()
 
     def forward(self, x):
@@ -75,7 +75,8 @@ class Experts(FeedForward):
         place = torch.empty(pairs, dtype=torch.int32, device=dev)
         ops.moe_scatter(sorted_in, place, x, chosen, weight, rank, seg)
         act = torch.empty((pairs, self.intermediate), dtype=x.dtype, device=dev)
-        ops.grouped_product(act, sorted_in, self.w_gate_up, epilogue="paired", segments=(seg, tiles), limit=self.limit)
+        ops.grouped_product(act, sorted_in, self.w_gate_up, epilogue="paired", segments=(seg, tiles), limit=self.limit,
+                            units=self.intermediate)
         results = torch.empty((pairs, self.hidden), dtype=torch.float32, device=dev)
         ops.grouped_product(results, act, self.w_down, segments=(seg, tiles))
         return ops.moe_combine(torch.empty((rows, self.hidden), dtype=torch.float32, device=dev), results, place)

@@ -210,11 +210,13 @@ def test_a_key_that_stands_out_shows_the_windows_edge():
 
 # ------------------------------------------------------------------------------ products with a weight per group
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("m,g,n,k", [(70, 3, 32, 16), (1, 5, 20, 24), (130, 2, 66, 70)])
-def test_a_product_per_head_on_strided_views(dtype, m, g, n, k):
+@pytest.mark.parametrize("m,g,n,k,pad", [(70, 3, 32, 16, 5), (1, 5, 20, 24, 8), (130, 2, 66, 70, 3), (300, 3, 136, 64, 16),
+                                         (17, 2, 24, 136, 0)])
+def test_a_product_per_head_on_strided_views(dtype, m, g, n, k, pad):
+    """(strides of x in multiples of 8 and bfloat16: the matrix-core kernel; all else the multiply-add kernel)"""
     from llmserve.ops import library as ops
 
-    x, w, z = rnd(m, g, k + 5, seed=41), rnd(g, n, k, seed=42, scale=0.3), rnd(m, 7 + g * n, seed=43)
+    x, w, z = rnd(m, g, k + pad, seed=41), rnd(g, n, k, seed=42, scale=0.3), rnd(m, 7 + g * n, seed=43)
     xd, wd = dev(x, dtype), dev(w, dtype)
     out = torch.full((m, g, n + 3), float("nan"), dtype=dtype, device=DEV)
     ops.grouped_product(out[:, :, :n], xd[:, :, :k], wd)
@@ -226,27 +228,36 @@ def test_a_product_per_head_on_strided_views(dtype, m, g, n, k):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("counts", [[5, 0, 70, 1], [0, 0, 3], [64, 64], [129]])
-def test_a_product_per_segment_of_rows(dtype, counts):
+@pytest.mark.parametrize("k,units", [(40, 24), (36, 70), (64, 32)])
+@pytest.mark.parametrize("counts", [[5, 0, 70, 1], [0, 0, 3], [64, 64], [129], [200, 1, 130]])
+def test_a_product_per_segment_of_rows(dtype, counts, k, units):
     from llmserve.ops import library as ops
 
-    g, k, n, limit = len(counts), 40, 24, 0.9
+    g, limit = len(counts), 0.9
     m = sum(counts)
-    seg = [0]
-    tiles = [0]
+    seg, tiles = [0], [[0], [0]]
     for c in counts:
         seg.append(seg[-1] + c)
-        tiles.append(tiles[-1] + -(-c // ops.GROUPED_TILE))
-    x, w = rnd(m, k, seed=51), rnd(g, 2 * n, k, seed=52, scale=0.3)
-    xd, wd = dev(x, dtype), dev(w, dtype)
-    out = torch.empty((m, 2 * n), dtype=torch.float32, device=DEV)
-    ops.grouped_product(out, xd, wd, segments=(ints(seg), ints(tiles)))
-    ref = torch.cat([xd[seg[e]: seg[e + 1]].double().cpu() @ wd[e].double().cpu().T for e in range(g)])
-    close(out, ref, dtype, "segments")
-    act = torch.empty((m, n), dtype=dtype, device=DEV)
-    ops.grouped_product(act, xd, wd, epilogue="paired", segments=(ints(seg), ints(tiles)), limit=limit)
-    ref = ref.to(dtype).double()
-    a, b = ref[:, 0::2].clamp(max=limit), ref[:, 1::2].clamp(min=-limit, max=limit)
+        tiles[0].append(tiles[0][-1] + -(-c // ops.GROUPED_TILE))
+        tiles[1].append(tiles[1][-1] + -(-c // ops.GROUPED_TILE_MFMA))
+    segments = (ints(seg), ints(tiles[0] + tiles[1]))
+    x, wa, wb = rnd(m, k, seed=51), rnd(g, units, k, seed=52, scale=0.3), rnd(g, units, k, seed=53, scale=0.3)
+    xd = dev(x, dtype)
+    wd = ops.stack_paired(dev(wa, dtype), dev(wb, dtype))
+    assert wd.shape == (g, 64 * -(-units // 32), k)
+    out = torch.empty((m, wd.shape[1]), dtype=torch.float32, device=DEV)
+    ops.grouped_product(out, xd, wd, segments=segments)
+    xs = xd.double().cpu()
+    ref_a = torch.cat([xs[seg[e]: seg[e + 1]] @ wa[e].to(dtype).double().T for e in range(g)])
+    ref_b = torch.cat([xs[seg[e]: seg[e + 1]] @ wb[e].to(dtype).double().T for e in range(g)])
+    first = min(32, units)
+    close(out[:, :first], ref_a[:, :first], dtype, "segments, first block of the first projection")
+    close(out[:, 32: 32 + first], ref_b[:, :first], dtype, "segments, first block of the second projection")
+    assert (out[:, first: 32] == 0).all()  # (rows of units that do not exist are zero)
+    act = torch.full((m, units), float("nan"), dtype=dtype, device=DEV)
+    ops.grouped_product(act, xd, wd, epilogue="paired", segments=segments, limit=limit, units=units)
+    a = ref_a.to(dtype).double().clamp(max=limit)
+    b = ref_b.to(dtype).double().clamp(min=-limit, max=limit)
     close(act, a * torch.sigmoid(1.702 * a) * (b + 1), dtype, "gated unit", loose=2)
 
 
@@ -304,12 +315,18 @@ def write_model(folder, config, seed):
 def logits_close(got, ref, dtype, what):
     """Per position: the difference of the logits (mean taken off, root mean square over the vocabulary) against the
     root mean square of the logits themselves.  32-bit: every position.  bfloat16: the median, and all but one
-    position in ten (a token whose choice of experts was a close call, and all that attend to it)."""
+    position in ten (a token whose choice of experts was a close call, and all that attend to it).  `got` and `ref`
+    may be lists of requests, which are then judged together."""
+    if isinstance(got, (list, tuple)):
+        scale = torch.cat([r.double().flatten() for r in ref]).pow(2).mean().sqrt()
+        got, ref = torch.cat(list(got)), torch.cat(list(ref))
+    else:
+        scale = ref.double().pow(2).mean().sqrt()
     got, ref = got.double(), ref.double()
     assert got.shape == ref.shape and torch.isfinite(got).all(), what
     d = got - ref
     d = d - d.mean(dim=-1, keepdim=True)
-    err = d.pow(2).mean(dim=-1).sqrt() / ref.pow(2).mean().sqrt()
+    err = d.pow(2).mean(dim=-1).sqrt() / scale
     worst = int(err.argmax())
     if dtype == torch.float32:
         assert float(err.max()) <= 5e-5, f"{what}: position {worst} is off by {float(err.max()):.2e}"
@@ -389,8 +406,7 @@ def test_every_way_of_cutting_gives_the_plain_logits(models, name, dtype_name, g
         assert runner._use_graphs == graphs  # every part of the model can be captured
         runner.storage.poison()
         got = run_trace(runner, steps)
-        for rid in seqs:
-            logits_close(got[rid], ref[rid], dtype, f"{name} {mode} {rid} {dtype_name}")
+        logits_close([got[rid] for rid in seqs], [ref[rid] for rid in seqs], dtype, f"{name} {mode} {dtype_name}")
         assert runner.manager.num_free_slots == 3
         assert all(a.num_free == pages for a in runner.manager.allocators.values())
         if graphs and mode == "decode":
@@ -511,7 +527,7 @@ def test_configurations_drawn_at_random(tmp_path, seed):
                                                                 max_num_seqs=3))
         runner.storage.poison()
         got = run_trace(runner, steps)
-        for rid in seqs:
-            logits_close(got[rid], ref[rid], getattr(torch, dtype_name), f"seed {seed} {rid} {dtype_name}: {config['layers']}")
+        logits_close([got[rid] for rid in seqs], [ref[rid] for rid in seqs], getattr(torch, dtype_name),
+                     f"seed {seed} {dtype_name}: {config['layers']}")
         assert runner.manager.num_free_slots == 3
         assert all(a.num_free == pages for a in runner.manager.allocators.values())
