@@ -25,7 +25,9 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_router_kernel(
         float dot = 0.f;
         for (int c = lane; c < hidden; c += LLMS_WAVE) dot = fmaf(to_f32(row[c]), to_f32(wr[c]), dot);
         dot = wave_sum(dot);
-        if (lane == 0) score[e] = 1.f / (1.f + expf(-dot));
+        // (a row that is not a number, as a padding row may be, gets a score like any other: every choice below must
+        // name an expert that exists)
+        if (lane == 0) score[e] = dot == dot ? 1.f / (1.f + expf(-dot)) : 0.f;
     }
     __syncthreads();
     if (wave != 0) return;
@@ -51,6 +53,7 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_router_kernel(
                 at = oa;
             }
         }
+        at = min(at, experts - 1);
         picked[k] = best;
         which[k] = at;
         sum += best;

@@ -1284,6 +1284,61 @@ def attend_latent(out: torch.Tensor, q: torch.Tensor, pool: torch.Tensor, block_
     return out
 
 
+LATENT_MFMA = os.environ.get("LLMSERVE_LATENT_ATTENTION", "") != "plain"  # "plain": keep the matrix-core kernel out
+LATENT_MFMA_PAIRS = 64  # (token, head) pairs of a workgroup of the matrix-core kernel
+LATENT_MFMA_KEYS = 32  # keys of one of its tiles
+
+
+def attend_latent_mfma_supported(dtype: torch.dtype, r: int, dr: int) -> bool:
+    """Whether the matrix-core kernel takes these sizes: bfloat16, r a multiple of 16 up to 512, r + dr a multiple of
+    8 that fits r's size class."""
+    if not LATENT_MFMA or dtype != torch.bfloat16 or r % 16 or (r + dr) % 8 or r > 512:
+        return False
+    padded = -(-(r + dr) // 32) * 32
+    return any(r <= 16 * rt and padded <= 32 * (rt // 2 + 2) for rt in (8, 16, 32))
+
+
+def attend_latent_mfma(out: torch.Tensor, q: torch.Tensor, pool: torch.Tensor, block_tables: torch.Tensor,
+                       cu_seqlens: torch.Tensor, context_lens: torch.Tensor, *, n_seqs: int, max_count: int, heads: int,
+                       r: int, dr: int, block_size: int, window: int, scale: float, splits: int = 1,
+                       table_rows: torch.Tensor | None = None) -> torch.Tensor:
+    """`attend_latent` on the matrix cores for the requests [0, n_seqs) of a step: request b owns the rows
+    cu_seqlens[b] .. cu_seqlens[b + 1] of q and out, which are its last tokens (positions context_lens[b] - count ..).
+    `max_count`: no request brings more rows.  `splits`: workgroups that share the keys of one block of rows."""
+    dev = _dev(out, q, pool, block_tables, cu_seqlens, context_lens, table_rows)
+    n = q.shape[0]
+    _rows(q, "q", heads * (r + dr))
+    _rows(out, "out", heads * r)
+    if not attend_latent_mfma_supported(q.dtype, r, dr):
+        raise ValueError(f"the matrix-core kernel does not take {q.dtype} rows of {r} + {dr}")
+    if out.shape[0] != n or out.dtype != q.dtype or pool.dtype != q.dtype:
+        raise ValueError("out, q and pool share one dtype; out and q their rows")
+    if not pool.is_contiguous() or pool.dim() != 4 or pool.shape[1] != 1 or pool.shape[2] != block_size or pool.shape[3] != r + dr:
+        raise ValueError(f"pool must be [pages, 1, {block_size}, {r + dr}], got {tuple(pool.shape)}")
+    if block_tables.dtype != torch.int32 or block_tables.dim() != 2 or not block_tables.is_contiguous():
+        raise ValueError("block_tables must be a contiguous int32 matrix")
+    _i32(cu_seqlens, "cu_seqlens")
+    _i32(context_lens, "context_lens")
+    if cu_seqlens.numel() < n_seqs + 1 or context_lens.numel() < n_seqs or n_seqs < 1 or max_count < 1:
+        raise ValueError("cu_seqlens and context_lens do not cover the requests")
+    if table_rows is not None:
+        _i32(table_rows, "table_rows")
+        if table_rows.numel() < n_seqs:
+            raise ValueError("table_rows does not cover the requests")
+    elif block_tables.shape[0] < n_seqs:
+        raise ValueError("fewer block tables than requests")
+    if window < 0 or not 1 <= splits <= 64:
+        raise ValueError("window must be >= 0 and splits 1 to 64")
+    if n == 0:
+        return out
+    ws = torch.empty(n * heads * splits * (r + 2), dtype=torch.float32, device=dev) if splits > 1 else None
+    _check(load("latent_mfma").llms_attend_latent_mfma(
+        _ptr(out), _ptr(q), _ptr(pool), _ptr(block_tables), c_int(block_tables.shape[1]), _ptr(table_rows), _ptr(cu_seqlens),
+        _ptr(context_lens), _ptr(ws), c_int(n_seqs), c_int(n), c_int(max_count), c_int(heads), c_int(r), c_int(dr),
+        c_int(block_size), c_int(window), c_float(scale), c_int(splits), _stream(dev)), "attend_latent_mfma")
+    return out
+
+
 # ------------------------------------------------------------------------------ products with a weight per group
 
 c_long = ctypes.c_long

@@ -69,6 +69,8 @@ class LatentAttention(Mixer):
         self.w_in = self.w_uq = self.w_absorb = self.w_uv = self.w_o = self.wq_norm = self.wc_norm = self.freq = None
 
     def libraries(self, dtype_name):
+        if dtype_name == "bfloat16" and ops.attend_latent_mfma_supported(torch.bfloat16, self.r, self.dr):
+            return ("latent", "grouped_gemm", "latent_mfma")
         return ("latent", "grouped_gemm")
 
     # ---- what it keeps between steps -------------------------------------------------------------
@@ -137,6 +139,23 @@ class LatentAttention(Mixer):
         return linear(out, self.w_o, out_dtype=torch.float32)
 
     def attend(self, out, folded, cache, view, batch):
-        ops.attend_latent(out, folded, cache.k_pool, view.block_tables, batch.token_seq, batch.positions,
-                          batch.context_lens, heads=self.heads, r=self.r, dr=self.dr, block_size=cache.block_size,
-                          window=int(self.window or 0), scale=self.scale, table_rows=batch.state_slots)
+        """out[n, a] = the softmax-weighted sum of the cache rows' latent parts for head a of token n: on the matrix
+        cores where the sizes allow (bfloat16), else by the kernel that takes any size and dtype."""
+        common = dict(heads=self.heads, r=self.r, dr=self.dr, block_size=cache.block_size, window=int(self.window or 0),
+                      scale=self.scale, table_rows=batch.state_slots)
+        if not ops.attend_latent_mfma_supported(folded.dtype, self.r, self.dr):
+            ops.attend_latent(out, folded, cache.k_pool, view.block_tables, batch.token_seq, batch.positions,
+                              batch.context_lens, **common)
+            return
+        splits = self.key_shares(batch.num_seqs, batch.max_count, batch.max_context, ops.compute_units(folded.device))
+        ops.attend_latent_mfma(out, folded, cache.k_pool, view.block_tables, batch.cu_seqlens, batch.context_lens,
+                               n_seqs=batch.num_seqs, max_count=batch.max_count, splits=splits, **common)
+
+    def key_shares(self, n_requests: int, max_new: int, max_context: int, cus: int = 256) -> int:
+        """Workgroups that share the keys of one block of 64 (token, head) pairs.  While the blocks alone leave
+        compute units idle (decoding, short portions), the tiles of 32 keys of each go to several workgroups, two
+        tiles a share at least, and a second kernel adds the shares up."""
+        blocks = n_requests * -(-max_new * self.heads // ops.LATENT_MFMA_PAIRS)
+        reach = max_context if self.window is None else min(max_context, self.window + max_new - 1)
+        tiles = -(-reach // ops.LATENT_MFMA_KEYS) + 1
+        return max(1, min(16, cus // max(blocks, 1), tiles // 2))

@@ -208,6 +208,61 @@ def test_a_key_that_stands_out_shows_the_windows_edge():
             close(got, attend_plain(q, rows, r, window, 1.0)[at], torch.float32, f"window {window} key {j}", loose=5)
 
 
+MFMA_CASES = [  # heads, r, dr, window, block size
+    (3, 32, 8, 11, 8), (6, 128, 16, 136, 16), (1, 16, 8, 1, 4), (5, 48, 40, None, 16), (16, 64, 32, 33, 8), (40, 32, 32, 70, 16),
+    (4, 256, 32, 50, 16), (2, 512, 64, 100, 16), (7, 144, 24, 64, 8),
+]
+
+
+@pytest.mark.parametrize("heads,r,dr,window,bs", MFMA_CASES)
+@pytest.mark.parametrize("splits", [1, 3])
+def test_matrix_core_attention_over_latent_rows(heads, r, dr, window, bs, splits):
+    """Several requests in one launch: portions of different lengths behind different prefixes, single tokens, a
+    request without keys; against the plain attention and, closely, against the kernel that takes any size."""
+    from llmserve.ops import library as ops
+
+    assert ops.attend_latent_mfma_supported(torch.bfloat16, r, dr)
+    dt = torch.bfloat16
+    lengths = [(150, 1), (97, 97), (200, 37), (64, 2), (33, 1), (300, 130)]  # (context after the step, tokens of the step)
+    scale = 0.5 / math.sqrt(r + dr)
+    pools, tables, qs, refs = [], [], [], []
+    for b, (ctx, count) in enumerate(lengths):
+        q, rows = rnd(ctx, heads, r + dr, seed=80 + b), rnd(ctx, r + dr, seed=90 + b)
+        refs.append(attend_plain(q.to(dt).double(), rows.to(dt).double(), r, window, scale)[ctx - count:])
+        qs.append(q[ctx - count:].reshape(count, -1))
+        pool, table = paged_rows(rows, bs, dt, seed=b)
+        pools.append(pool)
+        tables.append(table[0].tolist())
+    base, width = [0], max(len(t) for t in tables)
+    for pool in pools:
+        base.append(base[-1] + pool.shape[0])
+    pool = torch.cat(pools)
+    table = torch.zeros((len(lengths) + 2, width), dtype=torch.int32)
+    order = [3, 0, 5, 1, 7, 2]  # (a request's row of the block tables is its state slot, not its place in the step)
+    for b, t in enumerate(tables):
+        table[order[b], : len(t)] = torch.tensor(t) + base[b]
+    counts = [c for _, c in lengths] + [4]  # the last request has no keys (padding rows of a captured step)
+    cu = [0]
+    for c in counts:
+        cu.append(cu[-1] + c)
+    q_all = torch.cat(qs + [rnd(4, heads * (r + dr), seed=99)])
+    n = q_all.shape[0]
+    out = torch.full((n, heads * r), float("nan"), dtype=dt, device=DEV)
+    args = dict(heads=heads, r=r, dr=dr, block_size=bs, window=window or 0, scale=scale, table_rows=ints(order + [4]))
+    ops.attend_latent_mfma(out, dev(q_all, dt), pool, table.to(DEV), ints(cu), ints([c for c, _ in lengths] + [0]),
+                           n_seqs=len(counts), max_count=max(counts), splits=splits, **args)
+    assert (out[cu[-2]:] == 0).all()
+    token_seq = [b for b, c in enumerate(counts) for _ in range(c)]
+    positions = [ctx - count + i for ctx, count in lengths for i in range(count)] + [0] * 4
+    other = torch.empty_like(out)
+    ops.attend_latent(other, dev(q_all, dt), pool, table.to(DEV), ints(token_seq), ints(positions),
+                      ints([c for c, _ in lengths] + [0]), **args)
+    for b in range(len(lengths)):
+        got = out[cu[b]: cu[b + 1]].view(-1, heads, r)
+        close(got, refs[b], dt, f"request {b}")
+        close(got, other[cu[b]: cu[b + 1]].view(-1, heads, r).double().cpu(), dt, f"request {b} against the plain kernel")
+
+
 # ------------------------------------------------------------------------------ products with a weight per group
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("m,g,n,k,pad", [(70, 3, 32, 16, 5), (1, 5, 20, 24, 8), (130, 2, 66, 70, 3), (300, 3, 136, 64, 16),
