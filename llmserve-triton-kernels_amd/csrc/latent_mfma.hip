@@ -7,8 +7,9 @@
 // in tiles of 32 that all waves share through LDS: the tile's rows as they lie, for S^T = K Q'^T
 // (v_mfma_f32_16x16x32_bf16: lane l holds K[key l%16][8 numbers from 8*(l/16)] and Q'[the same numbers][pair l%16]; the
 // result holds S^T[key 4*(l/16) + i][pair l%16], i = 0..3), and their c-parts transposed, for O^T = C^T P^T
-// (v_mfma_f32_16x16x16_bf16: lane l holds C^T[number l%16][keys 4*(l/16) ..+3], one 8-byte read of the transposed tile,
-// and P^T[those keys][pair l%16], which is what the first product left in the lane).  A lane therefore keeps one pair's
+// (the same instruction, a tile being one step of 32 keys: lane l holds C^T[number l%16][keys 4*(l/16) ..+3 of both
+// halves of the tile], two 8-byte reads of the transposed tile, and P^T[those keys][pair l%16], which is what the first
+// product left in the lane).  A lane therefore keeps one pair's
 // column throughout: its maximum, its sum and its window are the lane's own.  Softmax in base 2, 32-bit.
 // The next tile's rows are fetched into registers while the present one is multiplied.
 //
@@ -20,7 +21,6 @@
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 lm_bf16x8;
-typedef __attribute__((ext_vector_type(4))) short lm_s16x4;
 typedef __attribute__((ext_vector_type(4))) float lm_f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t lm_u32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t lm_u32x2;
@@ -104,6 +104,16 @@ __global__ __launch_bounds__(LM_THREADS) void attend_latent_mfma_kernel(LatentAr
     // A thread's pieces of a tile: piece id = (piece / 2, key, piece % 2), so that the lanes of a wave hold 32 keys of
     // two neighbouring pieces: their 2-byte stores into the transposed tile fall into different banks, and the four
     // waves together read 128 contiguous bytes of every row.
+    // (page ids are looked up a tile ahead of the rows they lead to, so that no tile waits for two loads in a row)
+    int pg[NCH];
+    auto lookup = [&](int tile) {
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int id = tid + i * LM_THREADS;
+            const int key = tile * LM_KEYS + ((id >> 1) & (LM_KEYS - 1));
+            pg[i] = (key >= lo_block && key <= hi_block) ? table[key / a.block_size] : 0;
+        }
+    };
     auto fetch = [&](int tile) {
 #pragma unroll
         for (int i = 0; i < NCH; ++i) {
@@ -112,10 +122,8 @@ __global__ __launch_bounds__(LM_THREADS) void attend_latent_mfma_kernel(LatentAr
             const int key = tile * LM_KEYS + key_in;
             const bool there = piece < cpk && key >= lo_block && key <= hi_block && piece * 8 < a.dk;
             lm_u32x4 v = zero4;
-            if (there) {
-                const int page = table[key / a.block_size];
-                v = *reinterpret_cast<const lm_u32x4*>(a.pool + ((size_t)page * a.block_size + key % a.block_size) * a.dk + piece * 8);
-            }
+            if (there)
+                v = *reinterpret_cast<const lm_u32x4*>(a.pool + ((size_t)pg[i] * a.block_size + key % a.block_size) * a.dk + piece * 8);
             pf[i] = v;
         }
     };
@@ -138,12 +146,17 @@ __global__ __launch_bounds__(LM_THREADS) void attend_latent_mfma_kernel(LatentAr
     };
 
     if (t_begin < t_end) {
+        lookup(t_begin);
         fetch(t_begin);
+        if (t_begin + 1 < t_end) lookup(t_begin + 1);
         stage();
     }
     __syncthreads();
     for (int tile = t_begin; tile < t_end; ++tile) {
-        if (tile + 1 < t_end) fetch(tile + 1);
+        if (tile + 1 < t_end) {
+            fetch(tile + 1);
+            if (tile + 2 < t_end) lookup(tile + 2);
+        }
         const int key0 = tile * LM_KEYS;
         if (w_any && key0 <= w_hi && key0 + LM_KEYS > w_lo) {
             lm_f32x4 s[2];
@@ -174,7 +187,9 @@ __global__ __launch_bounds__(LM_THREADS) void attend_latent_mfma_kernel(LatentAr
             const float m_new = fmaxf(m, top);
             const bool some = m_new > -INFINITY;
             const float fix = some ? __builtin_amdgcn_exp2f(m - m_new) : 1.f;
-            lm_u32x2 pw[2];
+            // the tile's 32 keys as one step of the 32-deep instruction: a lane's 8 keys are the 4 it holds of each
+            // half of the tile (the order of keys within a step is free as long as both operands agree)
+            lm_u32x4 pw;
             float add = 0.f;
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
@@ -184,7 +199,8 @@ __global__ __launch_bounds__(LM_THREADS) void attend_latent_mfma_kernel(LatentAr
                     p[i] = some ? __builtin_amdgcn_exp2f(s[h][i] - m_new) : 0.f;
                     add += p[i];
                 }
-                pw[h] = (lm_u32x2){pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3])};
+                pw[2 * h] = pack_bf16x2(p[0], p[1]);
+                pw[2 * h + 1] = pack_bf16x2(p[2], p[3]);
             }
             l = l * fix + add;
             m = m_new;
@@ -197,12 +213,11 @@ __global__ __launch_bounds__(LM_THREADS) void attend_latent_mfma_kernel(LatentAr
 #pragma unroll
             for (int t = 0; t < RT; ++t) {
                 if (t < rt) {
-#pragma unroll
-                    for (int h = 0; h < 2; ++h) {
-                        const lm_u32x2 cf = *reinterpret_cast<const lm_u32x2*>(&ct[(16 * t + l16) * LM_CLD + 16 * h + 4 * quad]);
-                        o[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(lm_s16x4, cf),
-                                                                        __builtin_bit_cast(lm_s16x4, pw[h]), o[t], 0, 0, 0);
-                    }
+                    const uint16_t* crow = &ct[(16 * t + l16) * LM_CLD + 4 * quad];
+                    const lm_u32x2 c0 = *reinterpret_cast<const lm_u32x2*>(crow), c1 = *reinterpret_cast<const lm_u32x2*>(crow + 16);
+                    const lm_u32x4 cf = {c0[0], c0[1], c1[0], c1[1]};
+                    o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lm_bf16x8, cf),
+                                                                   __builtin_bit_cast(lm_bf16x8, pw), o[t], 0, 0, 0);
                 }
             }
         }
@@ -234,24 +249,35 @@ __global__ __launch_bounds__(LM_THREADS) void attend_latent_mfma_kernel(LatentAr
                 (lm_u32x2){pack_bf16x2(o[t][0] * inv, o[t][1] * inv), pack_bf16x2(o[t][2] * inv, o[t][3] * inv)};
 }
 
-// grid: (token, head) pairs; adds the shares up in their order
-__global__ __launch_bounds__(64) void latent_merge_kernel(bf16* __restrict__ out, const float* __restrict__ ws, int r, int splits) {
+// grid: (token, head) pairs; adds the shares up in their order.  Every thread reads the shares' maxima and sums at
+// once (all loads asked for before the first is used), then its numbers of every share.
+#define LM_MAX_SPLITS 16
+__global__ __launch_bounds__(256) void latent_merge_kernel(bf16* __restrict__ out, const float* __restrict__ ws, int r, int splits) {
     const size_t row = blockIdx.x;
     const float* shares = ws + row * splits * (r + 2);
+    float mz[LM_MAX_SPLITS], lz[LM_MAX_SPLITS];
+#pragma unroll
+    for (int z = 0; z < LM_MAX_SPLITS; ++z) {
+        mz[z] = z < splits ? shares[(size_t)z * (r + 2) + r] : -INFINITY;
+        lz[z] = z < splits ? shares[(size_t)z * (r + 2) + r + 1] : 0.f;
+    }
     float top = -INFINITY;
-    for (int z = 0; z < splits; ++z) top = fmaxf(top, shares[(size_t)z * (r + 2) + r]);
+#pragma unroll
+    for (int z = 0; z < LM_MAX_SPLITS; ++z) top = fmaxf(top, mz[z]);
     float total = 0.f;
-    for (int z = 0; z < splits; ++z) {
-        const float mz = shares[(size_t)z * (r + 2) + r];
-        total += mz > -INFINITY ? shares[(size_t)z * (r + 2) + r + 1] * __builtin_amdgcn_exp2f(mz - top) : 0.f;
+#pragma unroll
+    for (int z = 0; z < LM_MAX_SPLITS; ++z) {
+        mz[z] = mz[z] > -INFINITY ? __builtin_amdgcn_exp2f(mz[z] - top) : 0.f;  // (from here on: the share's factor)
+        total += lz[z] * mz[z];
     }
     const float inv = total > 0.f ? 1.f / total : 0.f;
-    for (int c = threadIdx.x; c < r; c += 64) {
+    for (int c = threadIdx.x; c < r; c += 256) {
+        float part[LM_MAX_SPLITS];
+#pragma unroll
+        for (int z = 0; z < LM_MAX_SPLITS; ++z) part[z] = z < splits ? shares[(size_t)z * (r + 2) + c] : 0.f;
         float v = 0.f;
-        for (int z = 0; z < splits; ++z) {
-            const float mz = shares[(size_t)z * (r + 2) + r];
-            if (mz > -INFINITY) v += shares[(size_t)z * (r + 2) + c] * __builtin_amdgcn_exp2f(mz - top);
-        }
+#pragma unroll
+        for (int z = 0; z < LM_MAX_SPLITS; ++z) v += mz[z] > 0.f ? part[z] * mz[z] : 0.f;
         out[row * r + c] = from_f32<bf16>(v * inv);
     }
 }
@@ -287,7 +313,7 @@ int llms_attend_latent_mfma(void* out, const void* q, const void* pool, const in
     LLMS_REQUIRE(rt != 0, "attend_latent_mfma: r a multiple of 16 up to 512, r + dr a multiple of 8 within the class");
     LLMS_REQUIRE(((uintptr_t)q % 16) == 0 && ((uintptr_t)pool % 16) == 0 && ((uintptr_t)out % 8) == 0,
                  "attend_latent_mfma: operands must be 16-byte aligned");
-    LLMS_REQUIRE(splits >= 1 && splits <= 64 && (splits == 1 || ws), "attend_latent_mfma: 1 to 64 shares, with their workspace");
+    LLMS_REQUIRE(splits >= 1 && splits <= LM_MAX_SPLITS && (splits == 1 || ws), "attend_latent_mfma: 1 to 16 shares, with their workspace");
     LatentArgs a;
     a.out = (bf16*)out, a.q = (const bf16*)q, a.pool = (const bf16*)pool, a.tables = tables, a.table_rows = table_rows;
     a.cu_seqlens = cu_seqlens, a.context_lens = context_lens, a.ws = ws;
@@ -302,7 +328,7 @@ int llms_attend_latent_mfma(void* out, const void* q, const void* pool, const in
                  : rt == 16 ? launch_latent<16>(a, grid, lds, stream)
                             : launch_latent<32>(a, grid, lds, stream);
     if (status != LLMS_OK) return status;
-    if (splits > 1) latent_merge_kernel<<<(unsigned)((size_t)n_rows * heads), 64, 0, stream>>>((bf16*)out, ws, r, splits);
+    if (splits > 1) latent_merge_kernel<<<(unsigned)((size_t)n_rows * heads), 256, 0, stream>>>((bf16*)out, ws, r, splits);
     LLMS_LAUNCH_CHECK();
 }
 

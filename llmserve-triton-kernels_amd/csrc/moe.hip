@@ -20,10 +20,33 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_router_kernel(
     extern __shared__ float score[];  // experts
     const int n = blockIdx.x, lane = threadIdx.x % LLMS_WAVE, wave = threadIdx.x / LLMS_WAVE;
     const T* row = h + (size_t)n * hidden;
+    const bool vec = hidden % (16 / sizeof(T)) == 0 && ((uintptr_t)h % 16) == 0 && ((uintptr_t)w_router % 16) == 0;
     for (int e = wave; e < experts; e += MOE_THREADS / LLMS_WAVE) {
         const T* wr = w_router + (size_t)e * hidden;
         float dot = 0.f;
-        for (int c = lane; c < hidden; c += LLMS_WAVE) dot = fmaf(to_f32(row[c]), to_f32(wr[c]), dot);
+        if (vec) {  // 16 bytes a lane and load, four loads in flight
+            constexpr int PER = 16 / sizeof(T);
+            typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+            for (int c0 = lane * PER; c0 < hidden; c0 += 4 * LLMS_WAVE * PER) {
+                u32x4 hv[4], wv[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int c = c0 + u * LLMS_WAVE * PER;
+                    const bool in = c < hidden;
+                    hv[u] = in ? *reinterpret_cast<const u32x4*>(row + c) : (u32x4){0, 0, 0, 0};
+                    wv[u] = in ? *reinterpret_cast<const u32x4*>(wr + c) : (u32x4){0, 0, 0, 0};
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const T* hp = reinterpret_cast<const T*>(&hv[u]);
+                    const T* wp = reinterpret_cast<const T*>(&wv[u]);
+#pragma unroll
+                    for (int k = 0; k < PER; ++k) dot = fmaf(to_f32(hp[k]), to_f32(wp[k]), dot);
+                }
+            }
+        } else {
+            for (int c = lane; c < hidden; c += LLMS_WAVE) dot = fmaf(to_f32(row[c]), to_f32(wr[c]), dot);
+        }
         dot = wave_sum(dot);
         // (a row that is not a number, as a padding row may be, gets a score like any other: every choice below must
         // name an expert that exists)

@@ -259,6 +259,99 @@ __global__ __launch_bounds__(S32_THREADS) void streams_norm_kernel(
     for (int c = threadIdx.x; c < hidden; c += S32_THREADS) orow[c] = from_f32<T>((u_row[c] - mean) * inv * weight[c]);
 }
 
+// The same for rows of a multiple of 4: a thread takes two float4 columns at a time with every load of both asked for
+// before the first is used, so a row of 2,048 costs one wait for memory.
+template <typename T>
+__global__ __launch_bounds__(S32_THREADS) void streams_norm_vec_kernel(
+    T* __restrict__ out, float* x_dst, const float* x_src, int src_broadcast, const float* __restrict__ y,
+    const float* __restrict__ mix, const float* __restrict__ wout, const float* __restrict__ read,
+    const float* __restrict__ weight, const int* __restrict__ rows, int streams, int hidden, float eps, int store) {
+    extern __shared__ float u_row[];
+    __shared__ float red[16];
+    __shared__ float coef[STREAMS_MAX * STREAMS_MAX + 2 * STREAMS_MAX];
+    const int r = blockIdx.x, n = rows ? rows[r] : r, S = streams, n4 = hidden / 4;
+    const float* src = x_src + (size_t)n * hidden * (src_broadcast ? 1 : S);
+    float* dst = x_dst + (size_t)n * hidden * S;
+    auto at = [](const float* p) { return *reinterpret_cast<const float4*>(p); };
+    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+    // the first columns are asked for before the coefficients are waited for
+    float4 xs[2][STREAMS_MAX], yv[2];
+    auto ask = [&](int base) {
+#pragma unroll
+        for (int v = 0; v < 2; ++v) {
+            const int c4 = base + v * S32_THREADS + threadIdx.x;
+#pragma unroll
+            for (int s = 0; s < STREAMS_MAX; ++s)
+                xs[v][s] = (s < S && c4 < n4) ? at(src + (src_broadcast ? 0 : (size_t)s * hidden) + 4 * c4) : zero;
+            yv[v] = (y && c4 < n4) ? at(y + (size_t)n * hidden + 4 * c4) : zero;
+        }
+    };
+    ask(0);
+    for (int i = threadIdx.x; i < S * S + 2 * S; i += S32_THREADS) {
+        float v;
+        if (i < S * S) v = mix ? mix[i] : (i / S == i % S ? 1.f : 0.f);
+        else if (i < S * S + S) v = wout ? wout[i - S * S] : 1.f;
+        else v = read ? read[i - S * S - S] : 1.f;
+        coef[i] = v;
+    }
+    __syncthreads();
+    const float* cm = coef;
+    const float* co = coef + S * S;
+    const float* cr = co + S;
+    float total = 0.f;
+    for (int base = 0; base < n4; base += 2 * S32_THREADS) {
+        if (base) ask(base);
+#pragma unroll
+        for (int v = 0; v < 2; ++v) {
+            const int c4 = base + v * S32_THREADS + threadIdx.x;
+            if (c4 >= n4) continue;
+            float4 u = zero;
+#pragma unroll
+            for (int t = 0; t < STREAMS_MAX; ++t) {
+                if (t < S) {
+                    float4 w4 = xs[v][t];
+                    if (y) {
+                        w4 = zero;
+#pragma unroll
+                        for (int s = 0; s < STREAMS_MAX; ++s)
+                            if (s < S) {
+                                const float k = cm[s * S + t];
+                                w4.x = fmaf(k, xs[v][s].x, w4.x), w4.y = fmaf(k, xs[v][s].y, w4.y);
+                                w4.z = fmaf(k, xs[v][s].z, w4.z), w4.w = fmaf(k, xs[v][s].w, w4.w);
+                            }
+                        const float k = co[t];
+                        w4.x = fmaf(k, yv[v].x, w4.x), w4.y = fmaf(k, yv[v].y, w4.y);
+                        w4.z = fmaf(k, yv[v].z, w4.z), w4.w = fmaf(k, yv[v].w, w4.w);
+                    }
+                    if (store) *reinterpret_cast<float4*>(dst + (size_t)t * hidden + 4 * c4) = w4;
+                    const float k = cr[t];
+                    u.x = fmaf(k, w4.x, u.x), u.y = fmaf(k, w4.y, u.y), u.z = fmaf(k, w4.z, u.z), u.w = fmaf(k, w4.w, u.w);
+                }
+            }
+            *reinterpret_cast<float4*>(u_row + 4 * c4) = u;
+            total += (u.x + u.y) + (u.z + u.w);
+        }
+    }
+    const float mean = block_sum(total, red) / (float)hidden;
+    float dev2 = 0.f;
+    for (int c4 = threadIdx.x; c4 < n4; c4 += S32_THREADS) {
+        const float4 u = *reinterpret_cast<const float4*>(u_row + 4 * c4);
+        const float a = u.x - mean, b = u.y - mean, c = u.z - mean, d = u.w - mean;
+        dev2 += (a * a + b * b) + (c * c + d * d);
+    }
+    const float inv = 1.0f / sqrtf(block_sum(dev2, red) / (float)hidden + eps);
+    if (!out) return;
+    T* orow = out + (size_t)r * hidden;
+    for (int c4 = threadIdx.x; c4 < n4; c4 += S32_THREADS) {
+        const float4 u = *reinterpret_cast<const float4*>(u_row + 4 * c4);
+        const float4 w4 = at(weight + 4 * c4);
+        orow[4 * c4 + 0] = from_f32<T>((u.x - mean) * inv * w4.x);
+        orow[4 * c4 + 1] = from_f32<T>((u.y - mean) * inv * w4.y);
+        orow[4 * c4 + 2] = from_f32<T>((u.z - mean) * inv * w4.z);
+        orow[4 * c4 + 3] = from_f32<T>((u.w - mean) * inv * w4.w);
+    }
+}
+
 extern "C" {
 
 int llms_embed_scale(int dtype, float* out, const void* table, const int* ids, int n, int hidden, int vocab, float scale,
@@ -346,16 +439,20 @@ int llms_streams_norm(int dtype, void* out, float* x_dst, const float* x_src, in
     LLMS_REQUIRE(x_src && (x_dst || !store) && (weight || !out), "streams_norm: a needed operand is missing");
     LLMS_REQUIRE((size_t)hidden * 4 <= 96 * 1024, "streams_norm: a row of up to 24,576 elements");
     const size_t lds = (size_t)hidden * sizeof(float);
-    if (lds > 32 * 1024) {
-        const void* kernel = dtype == 0 ? (const void*)streams_norm_kernel<float> : (const void*)streams_norm_kernel<bf16>;
-        LLMS_HIP_CHECK(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    }
-    if (dtype == 0)
-        streams_norm_kernel<float><<<n_out, S32_THREADS, lds, stream>>>((float*)out, x_dst, x_src, src_broadcast, y, mix, wout,
-                                                                        read, weight, rows, streams, hidden, eps, store);
-    else
-        streams_norm_kernel<bf16><<<n_out, S32_THREADS, lds, stream>>>((bf16*)out, x_dst, x_src, src_broadcast, y, mix, wout,
-                                                                       read, weight, rows, streams, hidden, eps, store);
+    auto aligned = [](const void* p) { return ((uintptr_t)p % 16) == 0; };
+    const bool vec = hidden % 4 == 0 && aligned(x_dst) && aligned(x_src) && aligned(y) && aligned(weight);
+#define STREAMS_GO(KERNEL, T)                                                                                               \
+    do {                                                                                                                    \
+        if (lds > 32 * 1024)                                                                                                \
+            LLMS_HIP_CHECK(hipFuncSetAttribute((const void*)KERNEL<T>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
+        KERNEL<T><<<n_out, S32_THREADS, lds, stream>>>((T*)out, x_dst, x_src, src_broadcast, y, mix, wout, read, weight, rows, \
+                                                       streams, hidden, eps, store);                                        \
+    } while (0)
+    if (vec && dtype == 0) STREAMS_GO(streams_norm_vec_kernel, float);
+    else if (vec) STREAMS_GO(streams_norm_vec_kernel, bf16);
+    else if (dtype == 0) STREAMS_GO(streams_norm_kernel, float);
+    else STREAMS_GO(streams_norm_kernel, bf16);
+#undef STREAMS_GO
     LLMS_LAUNCH_CHECK();
 }
 

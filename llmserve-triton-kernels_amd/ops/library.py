@@ -1327,8 +1327,8 @@ def attend_latent_mfma(out: torch.Tensor, q: torch.Tensor, pool: torch.Tensor, b
             raise ValueError("table_rows does not cover the requests")
     elif block_tables.shape[0] < n_seqs:
         raise ValueError("fewer block tables than requests")
-    if window < 0 or not 1 <= splits <= 64:
-        raise ValueError("window must be >= 0 and splits 1 to 64")
+    if window < 0 or not 1 <= splits <= 16:
+        raise ValueError("window must be >= 0 and splits 1 to 16")
     if n == 0:
         return out
     ws = torch.empty(n * heads * splits * (r + 2), dtype=torch.float32, device=dev) if splits > 1 else None
