@@ -136,7 +136,7 @@ template <typename TOut, int EPI>
 __global__ __launch_bounds__(256) void grouped_mfma_kernel(
     TOut* __restrict__ out, long out_ld, long out_gs, const bf16* __restrict__ x, long x_ld, long x_gs,
     const bf16* __restrict__ w, int M, int N, int K, int G, const int* __restrict__ seg, const int* __restrict__ tile_start,
-    const float* __restrict__ z, long z_ld, long z_gs, float limit, int units) {
+    const float* __restrict__ z, long z_ld, long z_gs, float limit, int units, int k_part, long part_stride) {
     __shared__ __attribute__((aligned(16))) uint16_t As[2][GM_BM * GM_LD];
     __shared__ __attribute__((aligned(16))) uint16_t Bs[2][GM_BN * GM_LD];
     int g, row0, row_end;
@@ -155,6 +155,7 @@ __global__ __launch_bounds__(256) void grouped_mfma_kernel(
     const int n0 = blockIdx.x * GM_BN;
     const bf16* xg = x + (seg ? 0 : (size_t)g * x_gs);
     const bf16* wg = w + (size_t)g * N * K;
+    const int w_ld = K;
     const int tid = threadIdx.x, wave = tid / LLMS_WAVE, lane = tid % LLMS_WAVE;
     const int wm = (wave % 2) * 64, wn = (wave / 2) * 64;
     const int l32 = lane % 32, hi = lane / 32;
@@ -176,7 +177,7 @@ __global__ __launch_bounds__(256) void grouped_mfma_kernel(
             const int k = k0 + ckc;
             const int am = row0 + crow[c], wr = n0 + crow[c];
             ra[c] = (am < row_end && k < K) ? *reinterpret_cast<const gg_u32x4*>(xg + (size_t)am * x_ld + k) : zero;
-            rb[c] = (wr < N && k < K) ? *reinterpret_cast<const gg_u32x4*>(wg + (size_t)wr * K + k) : zero;
+            rb[c] = (wr < N && k < K) ? *reinterpret_cast<const gg_u32x4*>(wg + (size_t)wr * w_ld + k) : zero;
         }
     };
     auto stage = [&](int buf) {
@@ -186,13 +187,18 @@ __global__ __launch_bounds__(256) void grouped_mfma_kernel(
             *reinterpret_cast<gg_u32x4*>(&Bs[buf][crow[c] * GM_LD + ckc]) = rb[c];
         }
     };
-    const int ktiles = (K + GM_BK - 1) / GM_BK;
-    fetch(0);
+    // (with segments the third grid dimension may share K out: part p takes k_part numbers from p * k_part on and
+    // leaves its sums in an array of its own, for the caller to add up)
+    const int k_begin = seg ? blockIdx.z * k_part : 0;
+    const int k_end = seg ? min(K, k_begin + k_part) : K;
+    const int ktiles = (k_end - k_begin + GM_BK - 1) / GM_BK;
+    K = k_end;
+    fetch(k_begin);
     stage(0);
     __syncthreads();
     for (int kt = 0; kt < ktiles; ++kt) {
         const int buf = kt & 1;
-        if (kt + 1 < ktiles) fetch((kt + 1) * GM_BK);
+        if (kt + 1 < ktiles) fetch(k_begin + (kt + 1) * GM_BK);
 #pragma unroll
         for (int s = 0; s < GM_BK / 16; ++s) {
             gg_bf16x8 af[2], bfr[2];
@@ -210,7 +216,7 @@ __global__ __launch_bounds__(256) void grouped_mfma_kernel(
         if (kt + 1 < ktiles) stage(buf ^ 1);
         __syncthreads();
     }
-    TOut* og = out + (seg ? 0 : (size_t)g * out_gs);
+    TOut* og = out + (seg ? (size_t)blockIdx.z * part_stride : (size_t)g * out_gs);
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
 #pragma unroll
@@ -237,10 +243,11 @@ __global__ __launch_bounds__(256) void grouped_mfma_kernel(
 template <typename TOut>
 static int launch_mfma(int epilogue, dim3 grid, hipStream_t stream, void* out, long out_ld, long out_gs, const void* x, long x_ld,
                        long x_gs, const void* w, int M, int N, int K, int G, const int* seg, const int* tile_start, const float* z,
-                       long z_ld, long z_gs, float limit, int units) {
+                       long z_ld, long z_gs, float limit, int units, int k_part, long part_stride) {
 #define GM_GO(EPI)                                                                                                          \
     grouped_mfma_kernel<TOut, EPI><<<grid, 256, 0, stream>>>((TOut*)out, out_ld, out_gs, (const bf16*)x, x_ld, x_gs,         \
-                                                             (const bf16*)w, M, N, K, G, seg, tile_start, z, z_ld, z_gs, limit, units)
+                                                             (const bf16*)w, M, N, K, G, seg, tile_start, z, z_ld, z_gs, limit, units, \
+                                                             k_part, part_stride)
     if (epilogue == GG_PLAIN) GM_GO(GG_PLAIN);
     else if (epilogue == GG_PAIRED) GM_GO(GG_PAIRED);
     else GM_GO(GG_GATED);
@@ -277,9 +284,12 @@ int llms_grouped_fma(int in_dtype, int out_dtype, int epilogue, void* out, long 
 }
 
 // The same on the matrix cores: bfloat16 operands, out_dtype 0 (float32) or 1 (bfloat16); tiles of 128 rows.
+// `k_parts` > 1 (segments, plain epilogue, float32 result): K is shared out to that many sets of workgroups, set p
+// leaving its sums at out + p * part_stride.
 int llms_grouped_mfma(int out_dtype, int epilogue, void* out, long out_ld, long out_gs, const void* x, long x_ld, long x_gs,
                       const void* w, int M, int N, int K, int G, const int* seg, const int* tile_start, int max_tiles,
-                      const float* z, long z_ld, long z_gs, float limit, int units, hipStream_t stream) {
+                      const float* z, long z_ld, long z_gs, float limit, int units, int k_parts, long part_stride,
+                      hipStream_t stream) {
     LLMS_REQUIRE(M > 0 && N > 0 && K > 0 && G > 0, "grouped_mfma: sizes must be positive");
     LLMS_REQUIRE(epilogue >= 0 && epilogue <= 2, "grouped_mfma: epilogue 0 (plain), 1 (paired) or 2 (gated)");
     LLMS_REQUIRE(epilogue != GG_PAIRED || (N % 64 == 0 && units > 0 && units <= N / 2),
@@ -288,14 +298,18 @@ int llms_grouped_mfma(int out_dtype, int epilogue, void* out, long out_ld, long 
     LLMS_REQUIRE((seg == nullptr) == (tile_start == nullptr), "grouped_mfma: segments come with their tile starts");
     LLMS_REQUIRE(K % 8 == 0 && x_ld % 8 == 0 && x_gs % 8 == 0, "grouped_mfma: K and the strides of x in multiples of 8");
     LLMS_REQUIRE(((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0, "grouped_mfma: x and w must be 16-byte aligned");
-    dim3 grid((N + GM_BN - 1) / GM_BN, seg ? max_tiles : (M + GM_BM - 1) / GM_BM, seg ? 1 : G);
+    LLMS_REQUIRE(k_parts >= 1 && k_parts <= 16, "grouped_mfma: 1 to 16 parts of K");
+    LLMS_REQUIRE(k_parts == 1 || (seg && epilogue == GG_PLAIN && out_dtype == 0),
+                 "grouped_mfma: K is shared out only with segments, the plain epilogue and a float32 result");
+    const int k_part = k_parts == 1 ? K : ((K + k_parts - 1) / k_parts + GM_BK - 1) / GM_BK * GM_BK;
+    dim3 grid((N + GM_BN - 1) / GM_BN, seg ? max_tiles : (M + GM_BM - 1) / GM_BM, seg ? k_parts : G);
     LLMS_REQUIRE(grid.y > 0 && grid.y <= 65535 && grid.z <= 65535, "grouped_mfma: too many rows or groups for one launch");
     if (out_dtype == 0)
         return launch_mfma<float>(epilogue, grid, stream, out, out_ld, out_gs, x, x_ld, x_gs, w, M, N, K, G, seg, tile_start, z, z_ld,
-                                  z_gs, limit, units);
+                                  z_gs, limit, units, k_part, part_stride);
     if (out_dtype == 1)
         return launch_mfma<bf16>(epilogue, grid, stream, out, out_ld, out_gs, x, x_ld, x_gs, w, M, N, K, G, seg, tile_start, z, z_ld,
-                                 z_gs, limit, units);
+                                 z_gs, limit, units, k_part, part_stride);
     LLMS_REQUIRE(false, "grouped_mfma: out_dtype must be 0 or 1");
 }
 

@@ -46,7 +46,7 @@ struct LatentArgs {
 template <int RT>
 __global__ __launch_bounds__(LM_THREADS) void attend_latent_mfma_kernel(LatentArgs a) {
     constexpr int QT = RT / 2 + 2;          // steps of 32 numbers of a query
-    constexpr int NCH = (LM_KEYS * QT * 4 + LM_THREADS - 1) / LM_THREADS;  // 16-byte pieces of a tile per thread
+    constexpr int NIT = (LM_KEYS / 2 * QT * 4 + LM_THREADS - 1) / LM_THREADS;  // pairs of 16-byte pieces of a tile per thread
     extern __shared__ __attribute__((aligned(16))) uint16_t lm_lds[];
     const int seq = blockIdx.y, split = blockIdx.z;
     const int first = a.cu_seqlens[seq], count = a.cu_seqlens[seq + 1] - first, ctx = a.context_lens[seq];
@@ -100,46 +100,55 @@ __global__ __launch_bounds__(LM_THREADS) void attend_latent_mfma_kernel(LatentAr
     float m = -INFINITY, l = 0.f;
     const int rt = a.r / 16, qt = a.dkp / 32, cpk = a.dkp / 8;  // (pieces of 8 numbers per key, padding included)
 
-    lm_u32x4 pf[NCH];
-    // A thread's pieces of a tile: piece id = (piece / 2, key, piece % 2), so that the lanes of a wave hold 32 keys of
-    // two neighbouring pieces: their 2-byte stores into the transposed tile fall into different banks, and the four
-    // waves together read 128 contiguous bytes of every row.
-    // (page ids are looked up a tile ahead of the rows they lead to, so that no tile waits for two loads in a row)
-    int pg[NCH];
+    // A thread's items of a tile: two neighbouring keys' 16-byte pieces at the same place of their rows, so that the
+    // transposed tile is written in whole words (a number of both keys).  Item id = (piece / 2, pair of keys, piece % 2):
+    // the lanes of a wave hold all 16 pairs of keys for four pieces, and their stores into the transposed tile fall
+    // into different banks.  Page ids are looked up a tile ahead of the rows they lead to, so that no tile waits for
+    // two loads in a row.
+    lm_u32x4 pf[NIT][2];
+    int pg[NIT][2];
     auto lookup = [&](int tile) {
 #pragma unroll
-        for (int i = 0; i < NCH; ++i) {
+        for (int i = 0; i < NIT; ++i) {
             const int id = tid + i * LM_THREADS;
-            const int key = tile * LM_KEYS + ((id >> 1) & (LM_KEYS - 1));
-            pg[i] = (key >= lo_block && key <= hi_block) ? table[key / a.block_size] : 0;
+            const int key = tile * LM_KEYS + 2 * ((id >> 1) & 15);
+#pragma unroll
+            for (int k = 0; k < 2; ++k)
+                pg[i][k] = (key + k >= lo_block && key + k <= hi_block) ? table[(key + k) / a.block_size] : 0;
         }
     };
     auto fetch = [&](int tile) {
 #pragma unroll
-        for (int i = 0; i < NCH; ++i) {
+        for (int i = 0; i < NIT; ++i) {
             const int id = tid + i * LM_THREADS;
-            const int key_in = (id >> 1) & (LM_KEYS - 1), piece = ((id >> 6) << 1) | (id & 1);
-            const int key = tile * LM_KEYS + key_in;
-            const bool there = piece < cpk && key >= lo_block && key <= hi_block && piece * 8 < a.dk;
-            lm_u32x4 v = zero4;
-            if (there)
-                v = *reinterpret_cast<const lm_u32x4*>(a.pool + ((size_t)pg[i] * a.block_size + key % a.block_size) * a.dk + piece * 8);
-            pf[i] = v;
+            const int piece = ((id >> 5) << 1) | (id & 1);
+            const int key = tile * LM_KEYS + 2 * ((id >> 1) & 15);
+#pragma unroll
+            for (int k = 0; k < 2; ++k) {
+                const bool there = piece < cpk && key + k >= lo_block && key + k <= hi_block && piece * 8 < a.dk;
+                lm_u32x4 v = zero4;
+                if (there)
+                    v = *reinterpret_cast<const lm_u32x4*>(
+                        a.pool + ((size_t)pg[i][k] * a.block_size + (key + k) % a.block_size) * a.dk + piece * 8);
+                pf[i][k] = v;
+            }
         }
     };
     auto stage = [&]() {
 #pragma unroll
-        for (int i = 0; i < NCH; ++i) {
+        for (int i = 0; i < NIT; ++i) {
             const int id = tid + i * LM_THREADS;
-            const int key_in = (id >> 1) & (LM_KEYS - 1), piece = ((id >> 6) << 1) | (id & 1);
+            const int piece = ((id >> 5) << 1) | (id & 1), key_in = 2 * ((id >> 1) & 15);
             if (piece >= cpk) continue;
-            *reinterpret_cast<lm_u32x4*>(&ks[key_in * kld + piece * 8]) = pf[i];
+            *reinterpret_cast<lm_u32x4*>(&ks[key_in * kld + piece * 8]) = pf[i][0];
+            *reinterpret_cast<lm_u32x4*>(&ks[(key_in + 1) * kld + piece * 8]) = pf[i][1];
             if (piece * 8 < a.r) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    const uint32_t two = pf[i][e];
-                    ct[(piece * 8 + 2 * e) * LM_CLD + key_in] = (uint16_t)(two & 0xffffu);
-                    ct[(piece * 8 + 2 * e + 1) * LM_CLD + key_in] = (uint16_t)(two >> 16);
+                    const uint32_t k0 = pf[i][0][e], k1 = pf[i][1][e];
+                    uint32_t* word = reinterpret_cast<uint32_t*>(&ct[(piece * 8 + 2 * e) * LM_CLD + key_in]);
+                    word[0] = (k0 & 0xffffu) | (k1 << 16);
+                    word[LM_CLD / 2] = (k0 >> 16) | (k1 & 0xffff0000u);
                 }
             }
         }

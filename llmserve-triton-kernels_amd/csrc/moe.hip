@@ -6,7 +6,8 @@
 //   moe_offsets   seg[e] = pairs of all experts before e, tile_start[e] = tiles of rows of all experts before e
 //   moe_scatter   rows sorted by expert: xs[seg[e] + rank] = weight * h[token] (the weight multiplies the expert's
 //                 input), rounded to T; place[pair] = that row
-//   moe_combine   y[n] = sum over the token's choices, in their order, of the experts' results rows (32-bit)
+//   moe_combine   y[n] = sum over the token's choices, in their order, of the experts' results rows (32-bit; a row may
+//                 arrive as partial sums over shares of the last product's K, added in the order of the shares)
 // A pair is p = token * top + choice.
 #include "common.h"
 
@@ -150,13 +151,17 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_scatter_kernel(
     for (int c = threadIdx.x; c < hidden; c += MOE_THREADS) dst[c] = from_f32<T>(wgt * to_f32(src[c]));
 }
 
-// grid: tokens
+// grid: tokens.  rows [parts, pairs, hidden]: a choice's result may arrive as several partial sums
 __global__ __launch_bounds__(MOE_THREADS) void moe_combine_kernel(float* __restrict__ y, const float* __restrict__ rows,
-                                                                  const int* __restrict__ place, int hidden, int top) {
+                                                                  const int* __restrict__ place, int hidden, int top,
+                                                                  int parts, long part_stride) {
     const int n = blockIdx.x;
     for (int c = threadIdx.x; c < hidden; c += MOE_THREADS) {
         float v = 0.f;
-        for (int k = 0; k < top; ++k) v += rows[(size_t)place[(size_t)n * top + k] * hidden + c];
+        for (int k = 0; k < top; ++k) {
+            const float* row = rows + (size_t)place[(size_t)n * top + k] * hidden + c;
+            for (int p = 0; p < parts; ++p) v += row[(size_t)p * part_stride];
+        }
         y[(size_t)n * hidden + c] = v;
     }
 }
@@ -201,9 +206,10 @@ int llms_moe_scatter(int dtype, void* xs, int* place, const void* h, const int* 
     LLMS_LAUNCH_CHECK();
 }
 
-int llms_moe_combine(float* y, const float* rows, const int* place, int n, int hidden, int top, hipStream_t stream) {
-    LLMS_REQUIRE(n > 0 && hidden > 0 && top > 0, "moe_combine: sizes must be positive");
-    moe_combine_kernel<<<n, MOE_THREADS, 0, stream>>>(y, rows, place, hidden, top);
+int llms_moe_combine(float* y, const float* rows, const int* place, int n, int hidden, int top, int parts, long part_stride,
+                     hipStream_t stream) {
+    LLMS_REQUIRE(n > 0 && hidden > 0 && top > 0 && parts > 0, "moe_combine: sizes must be positive");
+    moe_combine_kernel<<<n, MOE_THREADS, 0, stream>>>(y, rows, place, hidden, top, parts, part_stride);
     LLMS_LAUNCH_CHECK();
 }
 

@@ -1370,7 +1370,7 @@ def _grouped_on_matrix_cores(x: torch.Tensor, w: torch.Tensor, x_ld: int, x_gs: 
 
 def grouped_product(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, *, epilogue: str = "plain",
                     segments: "tuple[torch.Tensor, torch.Tensor] | None" = None, gate: torch.Tensor | None = None,
-                    gate_column: int = 0, limit: float = 0.0, units: int = 0) -> torch.Tensor:
+                    gate_column: int = 0, limit: float = 0.0, units: int = 0, k_parts: int = 1) -> torch.Tensor:
     """w [G, N, K].  Without `segments` every row meets every group: x [M, G, K] and out [M, G, N'] (views whose
     last axis has unit stride; the strides of the other two are free), out[m, g] = x[m, g] w[g]^T.  With `segments`
     = (seg [G + 1], tile_start [2, G + 1]) on the device (what `moe_sort` returns), x [M, K] and out [M, N'] hold rows
@@ -1379,7 +1379,13 @@ def grouped_product(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, *, epil
     out = min(a, limit) sigmoid(1.702 min(a, limit)) (clamp(b, +-limit) + 1)); "gated" (out times
     sigmoid(gate[m, gate_column + g N + n]), gate float32 [M, columns]).
     bfloat16 operands with K and the strides of x in multiples of 8 go to the matrix cores, all else to the 32-bit
-    multiply-add kernel."""
+    multiply-add kernel.  `k_parts` > 1 (as `grouped_k_parts` allows): out is float32 [k_parts, M, N] and holds partial
+    sums over shares of K, for the caller to add up."""
+    parts_out = None
+    if k_parts > 1:
+        if out.dim() != 3 or out.shape[0] != k_parts or not out.is_contiguous() or out.dtype != torch.float32:
+            raise ValueError("partial sums go to a contiguous float32 [k_parts, M, N] tensor")
+        parts_out, out = out, out[0]
     dev = _dev(out, x, w, gate, *(segments or ()))
     if w.dim() != 3 or not w.is_contiguous():
         raise ValueError("w must be a contiguous [G, N, K] tensor")
@@ -1410,6 +1416,8 @@ def grouped_product(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, *, epil
         m = x.shape[0]
         x_ld, x_gs, out_ld, out_gs = x.stride(0), 0, out.stride(0), 0
     mfma = _grouped_on_matrix_cores(x, w, x_ld, x_gs)
+    if k_parts > 1 and not (mfma and segments is not None and epilogue == "plain"):
+        raise ValueError("K is shared out only by the matrix-core kernel, with segments and the plain epilogue")
     seg_ptr = tiles_ptr = None
     max_tiles = 0
     if segments is not None:
@@ -1431,10 +1439,22 @@ def grouped_product(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, *, epil
               c_float(limit), c_int(units), _stream(dev))
     lib = load("grouped_gemm")
     if mfma:
-        _check(lib.llms_grouped_mfma(c_int(_code(out)), c_int(_EPILOGUES[epilogue]), *common), "grouped_product")
+        _check(lib.llms_grouped_mfma(c_int(_code(out)), c_int(_EPILOGUES[epilogue]), *common[:-1], c_int(k_parts),
+                                     c_long(out.numel() if k_parts > 1 else 0), common[-1]), "grouped_product")
     else:
         _check(lib.llms_grouped_fma(c_int(_code(x)), c_int(_code(out)), c_int(_EPILOGUES[epilogue]), *common), "grouped_product")
-    return out
+    return out if parts_out is None else parts_out
+
+
+def grouped_k_parts(x: torch.Tensor, w: torch.Tensor, cus: int = 256) -> int:
+    """Into how many shares a product over segments of few rows (x [M, K] against w [G, N, K]) splits its K: while the
+    weights' tiles alone leave compute units idle and each would walk a long K with one load in flight, up to 4 shares
+    of 512 numbers at least.  1 where the matrix-core kernel does not apply or the rows are many."""
+    g, n, k = w.shape
+    if x.shape[0] > 256 or not _grouped_on_matrix_cores(x, w, x.stride(0), 0):
+        return 1
+    tiles = g * -(-n // GROUPED_TILE_MFMA)
+    return max(1, min(4, cus // max(tiles, 1), k // 512))
 
 
 # ------------------------------------------------------------------------------ routing to experts
@@ -1504,17 +1524,20 @@ def moe_scatter(xs: torch.Tensor, place: torch.Tensor, h: torch.Tensor, chosen: 
 
 
 def moe_combine(y: torch.Tensor, rows: torch.Tensor, place: torch.Tensor) -> torch.Tensor:
-    """y[n] = sum_k rows[place[n, k]] in the order of k; y float32 [N, hidden], rows float32 [pairs, hidden]."""
+    """y[n] = sum_k rows[place[n, k]] in the order of k; y float32 [N, hidden], rows float32 [pairs, hidden] or
+    [parts, pairs, hidden] (partial sums of each row, added in the order of the parts)."""
     dev = _dev(y, rows, place)
     n, hidden = y.shape
     _f32(y, "y")
     _f32(rows, "rows")
-    _i32(place, "place", rows.shape[0])
-    top = rows.shape[0] // max(n, 1)
-    if rows.shape[1] != hidden or top * n != rows.shape[0]:
+    parts = rows.shape[0] if rows.dim() == 3 else 1
+    pairs = rows.shape[-2]
+    _i32(place, "place", pairs)
+    top = pairs // max(n, 1)
+    if rows.shape[-1] != hidden or top * n != pairs:
         raise ValueError("rows has top rows of y's width per row of y")
     if n == 0:
         return y
-    _check(load("moe").llms_moe_combine(_ptr(y), _ptr(rows), _ptr(place), c_int(n), c_int(hidden), c_int(top), _stream(dev)),
-           "moe_combine")
+    _check(load("moe").llms_moe_combine(_ptr(y), _ptr(rows), _ptr(place), c_int(n), c_int(hidden), c_int(top), c_int(parts),
+                                        c_long(pairs * hidden), _stream(dev)), "moe_combine")
     return y

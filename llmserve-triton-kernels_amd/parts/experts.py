@@ -77,6 +77,9 @@ class Experts(FeedForward):
         act = torch.empty((pairs, self.intermediate), dtype=x.dtype, device=dev)
         ops.grouped_product(act, sorted_in, self.w_gate_up, epilogue="paired", segments=(seg, tiles), limit=self.limit,
                             units=self.intermediate)
-        results = torch.empty((pairs, self.hidden), dtype=torch.float32, device=dev)
-        ops.grouped_product(results, act, self.w_down, segments=(seg, tiles))
+        # (few rows: the last product's K is shared out, and the sum over a token's choices adds the shares up as well)
+        parts = ops.grouped_k_parts(act, self.w_down, ops.compute_units(dev))
+        shape = (pairs, self.hidden) if parts == 1 else (parts, pairs, self.hidden)
+        results = torch.empty(shape, dtype=torch.float32, device=dev)
+        ops.grouped_product(results, act, self.w_down, segments=(seg, tiles), k_parts=parts)
         return ops.moe_combine(torch.empty((rows, self.hidden), dtype=torch.float32, device=dev), results, place)

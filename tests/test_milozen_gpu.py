@@ -316,6 +316,29 @@ def test_a_product_per_segment_of_rows(dtype, counts, k, units):
     close(act, a * torch.sigmoid(1.702 * a) * (b + 1), dtype, "gated unit", loose=2)
 
 
+@pytest.mark.parametrize("k,parts", [(64, 2), (200, 3), (1024, 4)])
+def test_shares_of_k_add_up_to_the_product(k, parts):
+    from llmserve.ops import library as ops
+
+    counts, n = [3, 0, 17, 1], 72
+    g, m = len(counts), sum(counts)
+    seg, tiles = [0], [[0], [0]]
+    for c in counts:
+        seg.append(seg[-1] + c)
+        tiles[0].append(tiles[0][-1] + -(-c // ops.GROUPED_TILE))
+        tiles[1].append(tiles[1][-1] + -(-c // ops.GROUPED_TILE_MFMA))
+    segments = (ints(seg), ints(tiles[0] + tiles[1]))
+    x, w = dev(rnd(m, k, seed=55), torch.bfloat16), dev(rnd(g, n, k, seed=56, scale=0.2), torch.bfloat16)
+    whole = ops.grouped_product(torch.empty((m, n), dtype=torch.float32, device=DEV), x, w, segments=segments)
+    shares = ops.grouped_product(torch.full((parts, m, n), float("nan"), dtype=torch.float32, device=DEV), x, w,
+                                 segments=segments, k_parts=parts)
+    close(shares.sum(0), whole.double().cpu(), torch.float32, "shares of K", loose=5)
+    place = ints(range(m))
+    y = ops.moe_combine(torch.empty((m, n), dtype=torch.float32, device=DEV), shares, place)
+    close(y, whole.double().cpu(), torch.float32, "added up by the sum over choices", loose=5)
+    assert ops.grouped_k_parts(x, w) == min(4, 256 // 4, k // 512) or k < 512
+
+
 # ------------------------------------------------------------------------------ experts
 def test_the_largest_scores_are_chosen_and_a_tie_goes_to_the_lower_expert():
     from llmserve.ops import library as ops
