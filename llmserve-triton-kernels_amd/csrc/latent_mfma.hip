@@ -3,7 +3,7 @@
 // q'[n, h] . row_j and sums the rows' c-parts.  All heads of a token meet the same rows: the (token, head) pairs of a
 // request are the columns of one product.
 //
-// A workgroup of 4 waves takes 64 consecutive (token, head) pairs of one request, a wave 16 of them, and walks the keys
+// A workgroup of 8 waves takes 128 consecutive (token, head) pairs of one request, a wave 16 of them, and walks the keys
 // in tiles of 32 that all waves share through LDS: the tile's rows as they lie, for S^T = K Q'^T
 // (v_mfma_f32_16x16x32_bf16: lane l holds K[key l%16][8 numbers from 8*(l/16)] and Q'[the same numbers][pair l%16]; the
 // result holds S^T[key 4*(l/16) + i][pair l%16], i = 0..3), and their c-parts transposed, for O^T = C^T P^T
@@ -25,8 +25,8 @@ typedef __attribute__((ext_vector_type(4))) float lm_f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t lm_u32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t lm_u32x2;
 
-#define LM_THREADS 256
-#define LM_PAIRS 64   // (token, head) pairs of a workgroup
+#define LM_THREADS 512
+#define LM_PAIRS 128  // (token, head) pairs of a workgroup
 #define LM_KEYS 32    // keys of a tile
 #define LM_CLD 40     // row stride of the transposed tile in elements: 32 keys + 8 of padding
 
@@ -40,6 +40,7 @@ struct LatentArgs {
     const int* context_lens;
     float* ws;            // shares: [N * H, splits, r + 2]
     int table_width, heads, r, dk, dkp, block_size, window, splits;
+    uint32_t page_magic;  // ceil(2^32 / block_size): key / block_size is the high word of key * page_magic (0: block_size is 1)
     float scale_log2;
 };
 
@@ -107,6 +108,7 @@ __global__ __launch_bounds__(LM_THREADS) void attend_latent_mfma_kernel(LatentAr
     // two loads in a row.
     lm_u32x4 pf[NIT][2];
     int pg[NIT][2];
+    auto page_of = [&](int key) { return a.page_magic ? (int)__umulhi((uint32_t)key, a.page_magic) : key; };
     auto lookup = [&](int tile) {
 #pragma unroll
         for (int i = 0; i < NIT; ++i) {
@@ -114,22 +116,22 @@ __global__ __launch_bounds__(LM_THREADS) void attend_latent_mfma_kernel(LatentAr
             const int key = tile * LM_KEYS + 2 * ((id >> 1) & 15);
 #pragma unroll
             for (int k = 0; k < 2; ++k)
-                pg[i][k] = (key + k >= lo_block && key + k <= hi_block) ? table[(key + k) / a.block_size] : 0;
+                pg[i][k] = (key + k >= lo_block && key + k <= hi_block) ? table[page_of(key + k)] : 0;
         }
     };
     auto fetch = [&](int tile) {
 #pragma unroll
         for (int i = 0; i < NIT; ++i) {
             const int id = tid + i * LM_THREADS;
-            const int piece = ((id >> 5) << 1) | (id & 1);
+            const int piece = ((id >> 5) << 1) | (id & 1);  // (32 pieces per round of the workgroup's 512 threads)
             const int key = tile * LM_KEYS + 2 * ((id >> 1) & 15);
 #pragma unroll
             for (int k = 0; k < 2; ++k) {
                 const bool there = piece < cpk && key + k >= lo_block && key + k <= hi_block && piece * 8 < a.dk;
                 lm_u32x4 v = zero4;
-                if (there)
+                if (there)  // (page * block_size + key % block_size, without a division)
                     v = *reinterpret_cast<const lm_u32x4*>(
-                        a.pool + ((size_t)pg[i][k] * a.block_size + (key + k) % a.block_size) * a.dk + piece * 8);
+                        a.pool + (size_t)((pg[i][k] - page_of(key + k)) * a.block_size + key + k) * a.dk + piece * 8);
                 pf[i][k] = v;
             }
         }
@@ -329,6 +331,7 @@ int llms_attend_latent_mfma(void* out, const void* q, const void* pool, const in
     a.table_width = table_width, a.heads = heads, a.r = r, a.dk = dk, a.dkp = (dk + 31) / 32 * 32;
     a.block_size = block_size, a.window = window, a.splits = splits;
     a.scale_log2 = scale * 1.4426950408889634f;
+    a.page_magic = block_size == 1 ? 0u : (uint32_t)(((1ull << 32) + block_size - 1) / block_size);
     const long long blocks = ((long long)max_count * heads + LM_PAIRS - 1) / LM_PAIRS;
     LLMS_REQUIRE(blocks < (1ll << 31) && n_seqs <= 65535, "attend_latent_mfma: too many workgroups for one launch");
     dim3 grid((unsigned)blocks, n_seqs, splits);

@@ -1285,7 +1285,7 @@ def attend_latent(out: torch.Tensor, q: torch.Tensor, pool: torch.Tensor, block_
 
 
 LATENT_MFMA = os.environ.get("LLMSERVE_LATENT_ATTENTION", "") != "plain"  # "plain": keep the matrix-core kernel out
-LATENT_MFMA_PAIRS = 64  # (token, head) pairs of a workgroup of the matrix-core kernel
+LATENT_MFMA_PAIRS = 128  # (token, head) pairs of a workgroup of the matrix-core kernel
 LATENT_MFMA_KEYS = 32  # keys of one of its tiles
 
 
