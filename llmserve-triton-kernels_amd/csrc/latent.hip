@@ -62,6 +62,26 @@ __global__ __launch_bounds__(LAT_THREADS) void latent_query_kernel(
     const int n = blockIdx.x, dq = dn + dr;
     const float position = (float)positions[n];
     const float* qr = q + (size_t)n * heads * dq;
+    if (dn % 2 == 0 && dr % 2 == 0) {  // a thread takes two neighbours: a pair of the rotation has one sine and cosine
+        const int half = dq / 2;
+        for (int i = threadIdx.x; i < heads * half; i += LAT_THREADS) {
+            const int h = i / half, e = 2 * (i - h * half);
+            const float a = qr[h * dq + e], b = qr[h * dq + e + 1];
+            if (e < dn) {
+                T* dst = plain + ((size_t)n * heads + h) * dn + e;
+                dst[0] = from_f32<T>(a), dst[1] = from_f32<T>(b);
+            } else {
+                T* dst = folded + ((size_t)n * heads + h) * (r + dr) + r + (e - dn);
+                float2 turned = make_float2(a, b);
+                if (e - dn < dims) {
+                    const float2 sc = rotary_angle(position, freq[(e - dn) >> 1]);
+                    turned = rotate_pair(a, b, sc.y, sc.x);
+                }
+                dst[0] = from_f32<T>(turned.x), dst[1] = from_f32<T>(turned.y);
+            }
+        }
+        return;
+    }
     for (int i = threadIdx.x; i < heads * dq; i += LAT_THREADS) {
         const int h = i / dq, e = i - h * dq;
         if (e < dn)

@@ -84,6 +84,10 @@ __global__ __launch_bounds__(LM_THREADS) void attend_latent_mfma_kernel(LatentAr
     const bool w_any = p0 + wave * 16 < pairs;
     const int w_lo = a.window > 0 ? max(0, start + w_first / a.heads - a.window + 1) : 0;
     const int w_hi = start + w_last / a.heads;
+    // keys [w_from, w_seen] are seen by every pair of the wave (none when some of its 16 columns hold no pair)
+    const bool w_full = p0 + wave * 16 + 15 < pairs;
+    const int w_seen = w_full ? start + w_first / a.heads : -1;
+    const int w_from = a.window > 0 ? max(0, w_hi - a.window + 1) : 0;
 
     const lm_u32x4 zero4 = {0, 0, 0, 0};
     lm_u32x4 qf[QT];
@@ -183,21 +187,28 @@ __global__ __launch_bounds__(LM_THREADS) void attend_latent_mfma_kernel(LatentAr
                     }
                 }
             }
+            // A tile that every pair of the wave sees whole is not compared key by key (uniform over the wave).
+            const bool whole = key0 + LM_KEYS - 1 <= w_seen && key0 >= w_from;
             float top = -INFINITY;
 #pragma unroll
             for (int h = 0; h < 2; ++h)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const int key = key0 + 16 * h + 4 * quad + i;
-                    const float v = (key <= pos && key >= lo) ? s[h][i] * a.scale_log2 : -INFINITY;
+                    float v = s[h][i] * a.scale_log2;
+                    if (!whole) v = (key <= pos && key >= lo) ? v : -INFINITY;
                     s[h][i] = v;
                     top = fmaxf(top, v);
                 }
             top = fmaxf(top, __shfl_xor(top, 16, LLMS_WAVE));
             top = fmaxf(top, __shfl_xor(top, 32, LLMS_WAVE));
-            const float m_new = fmaxf(m, top);
+            // The weights are taken against a reference that follows the maximum only when some pair's maximum has
+            // passed it by more than 2^8 (the quotient at the end does not depend on the reference): the sums are
+            // rescaled in few tiles.
+            const bool moved = __any(top > m + 8.f);
+            const float m_new = moved ? fmaxf(m, top) : m;
             const bool some = m_new > -INFINITY;
-            const float fix = some ? __builtin_amdgcn_exp2f(m - m_new) : 1.f;
+            const float fix = (moved && some) ? __builtin_amdgcn_exp2f(m - m_new) : 1.f;
             // the tile's 32 keys as one step of the 32-deep instruction: a lane's 8 keys are the 4 it holds of each
             // half of the tile (the order of keys within a step is free as long as both operands agree)
             lm_u32x4 pw;
@@ -215,8 +226,7 @@ __global__ __launch_bounds__(LM_THREADS) void attend_latent_mfma_kernel(LatentAr
             }
             l = l * fix + add;
             m = m_new;
-            // (pairs whose maximum did not move keep their sums as they are: uniform over the wave only if none moved)
-            if (__any(fix != 1.f)) {
+            if (moved) {
 #pragma unroll
                 for (int t = 0; t < RT; ++t)
                     if (t < rt) o[t] = o[t] * fix;

@@ -156,6 +156,27 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_combine_kernel(float* __restr
                                                                   const int* __restrict__ place, int hidden, int top,
                                                                   int parts, long part_stride) {
     const int n = blockIdx.x;
+    if (hidden % 4 == 0 && part_stride % 4 == 0 && ((uintptr_t)rows % 16) == 0 && ((uintptr_t)y % 16) == 0) {
+        // 16 bytes a thread and load, the loads of four summands in flight together
+        for (int c = 4 * threadIdx.x; c < hidden; c += 4 * MOE_THREADS) {
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            const int terms = top * parts;
+            for (int t0 = 0; t0 < terms; t0 += 4) {
+                float4 part[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int t = t0 + u, k = t / parts, p = t - k * parts;
+                    part[u] = t < terms ? *reinterpret_cast<const float4*>(rows + (size_t)place[(size_t)n * top + k] * hidden +
+                                                                           (size_t)p * part_stride + c)
+                                        : make_float4(0.f, 0.f, 0.f, 0.f);
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) v.x += part[u].x, v.y += part[u].y, v.z += part[u].z, v.w += part[u].w;
+            }
+            *reinterpret_cast<float4*>(y + (size_t)n * hidden + c) = v;
+        }
+        return;
+    }
     for (int c = threadIdx.x; c < hidden; c += MOE_THREADS) {
         float v = 0.f;
         for (int k = 0; k < top; ++k) {
