@@ -119,7 +119,9 @@ static int launch_fma(int epilogue, dim3 grid, hipStream_t stream, void* out, lo
 }
 
 // ------------------------------------------------------------------------------ bfloat16 on the matrix cores
-// 128 x 128 tiles through double-buffered LDS, 4 waves of 64 x 64, v_mfma_f32_32x32x16_bf16: lane l holds
+// 128 x 128 tiles, 64 of K at a time, through double-buffered LDS (72 KB: two workgroups a compute unit; a tile of
+// K in flight is 32 KB a workgroup, which is what lets few rows stream the weights near the memory's rate), 4 waves of
+// 64 x 64, v_mfma_f32_32x32x16_bf16: lane l holds
 // A[i = l%32][k = 8*(l/32) .. +7] and B[k = same][j = l%32]; result D[i = 8*(r/4) + 4*(l/32) + r%4][j = l%32].
 // Here i = row m and j = weight row n, so a wave's two column blocks of 32 are the a and b rows of the same 32 units
 // of a paired weight (columns 0..31 and 32..63 of its 64), both in the same lane.
@@ -129,16 +131,19 @@ typedef __attribute__((ext_vector_type(4))) uint32_t gg_u32x4;
 
 #define GM_BM 128
 #define GM_BN 128
-#define GM_BK 32
-#define GM_LD 40  // LDS row stride in elements: 32 + 8 of padding against bank conflicts
+#define GM_BK 64
+#define GM_LD 72  // LDS row stride in elements: 64 + 8 of padding against bank conflicts
+#define GM_PIECES (GM_BM * GM_BK / 8 / 256)  // 16-byte pieces of an operand tile per thread
+#define GM_LDS_BYTES (2 * 2 * GM_BM * GM_LD * 2)  // two buffers of two operand tiles
 
 template <typename TOut, int EPI>
 __global__ __launch_bounds__(256) void grouped_mfma_kernel(
     TOut* __restrict__ out, long out_ld, long out_gs, const bf16* __restrict__ x, long x_ld, long x_gs,
     const bf16* __restrict__ w, int M, int N, int K, int G, const int* __restrict__ seg, const int* __restrict__ tile_start,
     const float* __restrict__ z, long z_ld, long z_gs, float limit, int units, int k_part, long part_stride) {
-    __shared__ __attribute__((aligned(16))) uint16_t As[2][GM_BM * GM_LD];
-    __shared__ __attribute__((aligned(16))) uint16_t Bs[2][GM_BN * GM_LD];
+    extern __shared__ __attribute__((aligned(16))) uint16_t gm_lds[];
+    uint16_t(*As)[GM_BM * GM_LD] = reinterpret_cast<uint16_t(*)[GM_BM * GM_LD]>(gm_lds);
+    uint16_t(*Bs)[GM_BN * GM_LD] = reinterpret_cast<uint16_t(*)[GM_BN * GM_LD]>(gm_lds + 2 * GM_BM * GM_LD);
     int g, row0, row_end;
     if (seg) {
         const int t = blockIdx.y;
@@ -167,24 +172,23 @@ __global__ __launch_bounds__(256) void grouped_mfma_kernel(
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-    // staging: 512 pieces of 8 elements per operand tile, two per thread
-    gg_u32x4 ra[2], rb[2];
-    const int crow[2] = {tid / 4, (tid + 256) / 4};
-    const int ckc = (tid % 4) * 8;
+    // staging: 1,024 pieces of 8 elements per operand tile, four per thread
+    gg_u32x4 ra[GM_PIECES], rb[GM_PIECES];
+    const int crow0 = tid / 8, ckc = (tid % 8) * 8;
     auto fetch = [&](int k0) {
 #pragma unroll
-        for (int c = 0; c < 2; ++c) {
+        for (int c = 0; c < GM_PIECES; ++c) {
             const int k = k0 + ckc;
-            const int am = row0 + crow[c], wr = n0 + crow[c];
+            const int am = row0 + crow0 + 32 * c, wr = n0 + crow0 + 32 * c;
             ra[c] = (am < row_end && k < K) ? *reinterpret_cast<const gg_u32x4*>(xg + (size_t)am * x_ld + k) : zero;
             rb[c] = (wr < N && k < K) ? *reinterpret_cast<const gg_u32x4*>(wg + (size_t)wr * w_ld + k) : zero;
         }
     };
     auto stage = [&](int buf) {
 #pragma unroll
-        for (int c = 0; c < 2; ++c) {
-            *reinterpret_cast<gg_u32x4*>(&As[buf][crow[c] * GM_LD + ckc]) = ra[c];
-            *reinterpret_cast<gg_u32x4*>(&Bs[buf][crow[c] * GM_LD + ckc]) = rb[c];
+        for (int c = 0; c < GM_PIECES; ++c) {
+            *reinterpret_cast<gg_u32x4*>(&As[buf][(crow0 + 32 * c) * GM_LD + ckc]) = ra[c];
+            *reinterpret_cast<gg_u32x4*>(&Bs[buf][(crow0 + 32 * c) * GM_LD + ckc]) = rb[c];
         }
     };
     // (with segments the third grid dimension may share K out: part p takes k_part numbers from p * k_part on and
@@ -245,12 +249,18 @@ static int launch_mfma(int epilogue, dim3 grid, hipStream_t stream, void* out, l
                        long x_gs, const void* w, int M, int N, int K, int G, const int* seg, const int* tile_start, const float* z,
                        long z_ld, long z_gs, float limit, int units, int k_part, long part_stride) {
 #define GM_GO(EPI)                                                                                                          \
-    grouped_mfma_kernel<TOut, EPI><<<grid, 256, 0, stream>>>((TOut*)out, out_ld, out_gs, (const bf16*)x, x_ld, x_gs,         \
+    LLMS_HIP_CHECK(hipFuncSetAttribute((const void*)grouped_mfma_kernel<TOut, EPI>,                                         \
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));                          \
+    grouped_mfma_kernel<TOut, EPI><<<grid, 256, GM_LDS_BYTES, stream>>>((TOut*)out, out_ld, out_gs, (const bf16*)x, x_ld, x_gs, \
                                                              (const bf16*)w, M, N, K, G, seg, tile_start, z, z_ld, z_gs, limit, units, \
                                                              k_part, part_stride)
-    if (epilogue == GG_PLAIN) GM_GO(GG_PLAIN);
-    else if (epilogue == GG_PAIRED) GM_GO(GG_PAIRED);
-    else GM_GO(GG_GATED);
+    if (epilogue == GG_PLAIN) {
+        GM_GO(GG_PLAIN);
+    } else if (epilogue == GG_PAIRED) {
+        GM_GO(GG_PAIRED);
+    } else {
+        GM_GO(GG_GATED);
+    }
 #undef GM_GO
     LLMS_LAUNCH_CHECK();
 }
